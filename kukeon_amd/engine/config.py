@@ -94,6 +94,9 @@ class EngineConfig:
                                     # the KV bandwidth, 2x the capacity)
     seed: int = 1234
     tp_size: int = 1
+    # slots of carried per-sequence state for models that have any
+    # (0 = one per session)
+    state_slots: int = 0
 
     @property
     def max_blocks_per_seq(self) -> int:

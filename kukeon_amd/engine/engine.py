@@ -22,13 +22,14 @@ from __future__ import annotations
 import logging
 import weakref
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
 from kukeon_amd import ops
 from kukeon_amd.engine.config import EngineConfig, ModelConfig, SamplingParams
-from kukeon_amd.engine.kv_cache import PagedKVCache, SequenceKV
+from kukeon_amd.engine.kv_cache import (LayeredKVCache, PagedKVCache,
+                                        SequenceKV, StatePool)
 from kukeon_amd.models.llama import AttnMeta
 
 log = logging.getLogger("kukeon.engine")
@@ -65,35 +66,68 @@ class LLMEngine:
         self.device = torch.device(device)
         self.is_cuda = self.device.type == "cuda"
         import kukeon_amd.parallel as parallel
-        self.hk = cfg.num_kv_heads // max(1, parallel.tp_size())
-        self.hq = cfg.num_q_heads // max(1, parallel.tp_size())
-
-        kv_torch_dtype = (torch.uint8 if ecfg.kv_dtype == "fp8"
+        # a model that states its own cache layout (per-layer shapes, pages
+        # shared between layers, carried state) gets a LayeredKVCache and a
+        # StatePool; the uniform Llama/Mixtral layout keeps the single
+        # [L, blocks, Hk, BS, D] pool
+        self.layered = hasattr(model, "kv_specs")
+        self.act_dtype = (model.activation_dtype()
+                          if hasattr(model, "activation_dtype")
                           else torch.bfloat16)
-        kv_bytes = 1 if ecfg.kv_dtype == "fp8" else 2
         nblocks = ecfg.num_kv_blocks
-        if nblocks <= 0:
-            if self.is_cuda:
-                free, _total = torch.cuda.mem_get_info(self.device)
-                # oversubscribed rehearsals (more local ranks than GPUs,
-                # e.g. a world-2 torchrun on a 1-GPU box) share the HBM:
-                # split the KV budget so the second rank isn't starved
-                import os as _os
-                lw = int(_os.environ.get("LOCAL_WORLD_SIZE", "1") or 1)
-                ndev = max(1, torch.cuda.device_count())
-                share = max(1, -(-lw // ndev))
-                budget = int(free * ecfg.kv_mem_fraction) // share - (2 << 30)
-                nblocks = PagedKVCache.blocks_from_bytes(
-                    max(budget, 1 << 28), cfg.num_layers, self.hk,
-                    ecfg.block_size, cfg.head_dim, dtype_bytes=kv_bytes)
-                nblocks = min(nblocks, 4_000_000)
-            else:
-                nblocks = 512
-        self.kv = PagedKVCache(cfg.num_layers, nblocks, self.hk,
-                               ecfg.block_size, cfg.head_dim, self.device,
-                               dtype=kv_torch_dtype)
-        log.info("KV cache: %d blocks (%.1f GiB for K+V)", nblocks,
-                 self.kv.k.nbytes * 2 / (1 << 30))
+        if self.layered:
+            specs = model.kv_specs()
+            self.hk = self.hq = 0
+            kv_bytes = torch.empty(0, dtype=self.act_dtype).element_size()
+            if nblocks <= 0:
+                if self.is_cuda:
+                    free, _total = torch.cuda.mem_get_info(self.device)
+                    budget = int(free * ecfg.kv_mem_fraction) - (2 << 30)
+                    nblocks = LayeredKVCache.blocks_from_bytes(
+                        max(budget, 1 << 28), specs, ecfg.block_size,
+                        dtype_bytes=kv_bytes)
+                    nblocks = min(nblocks, 4_000_000)
+                else:
+                    nblocks = 512
+            self.kv = LayeredKVCache(specs, nblocks, ecfg.block_size,
+                                     self.device, dtype=self.act_dtype)
+            log.info("KV cache: %d blocks (%.2f GiB for K+V)", nblocks,
+                     self.kv.nbytes / (1 << 30))
+        else:
+            self.hk = cfg.num_kv_heads // max(1, parallel.tp_size())
+            self.hq = cfg.num_q_heads // max(1, parallel.tp_size())
+            kv_torch_dtype = (torch.uint8 if ecfg.kv_dtype == "fp8"
+                              else torch.bfloat16)
+            kv_bytes = 1 if ecfg.kv_dtype == "fp8" else 2
+            if nblocks <= 0:
+                if self.is_cuda:
+                    free, _total = torch.cuda.mem_get_info(self.device)
+                    # oversubscribed rehearsals (more local ranks than GPUs,
+                    # e.g. a world-2 torchrun on a 1-GPU box) share the HBM:
+                    # split the KV budget so the second rank isn't starved
+                    import os as _os
+                    lw = int(_os.environ.get("LOCAL_WORLD_SIZE", "1") or 1)
+                    ndev = max(1, torch.cuda.device_count())
+                    share = max(1, -(-lw // ndev))
+                    budget = int(free * ecfg.kv_mem_fraction) // share - \
+                        (2 << 30)
+                    nblocks = PagedKVCache.blocks_from_bytes(
+                        max(budget, 1 << 28), cfg.num_layers, self.hk,
+                        ecfg.block_size, cfg.head_dim, dtype_bytes=kv_bytes)
+                    nblocks = min(nblocks, 4_000_000)
+                else:
+                    nblocks = 512
+            self.kv = PagedKVCache(cfg.num_layers, nblocks, self.hk,
+                                   ecfg.block_size, cfg.head_dim, self.device,
+                                   dtype=kv_torch_dtype)
+            log.info("KV cache: %d blocks (%.1f GiB for K+V)", nblocks,
+                     self.kv.k.nbytes * 2 / (1 << 30))
+        # carried per-sequence state (convolution tails, recurrences)
+        self.states: Optional[StatePool] = None
+        if hasattr(model, "state_shapes"):
+            nslots = ecfg.state_slots or ecfg.max_sessions
+            self.states = StatePool(model.state_shapes(), nslots,
+                                    self.device)
 
         self.waiting: List[Request] = []
         self._next_id = 0
@@ -115,6 +149,12 @@ class LLMEngine:
         self.d_slots = torch.full((self.Bmax,), -1, dtype=torch.int32, device=d)
         self.d_bt = torch.zeros(self.Bmax, mb, dtype=torch.int32, device=d)
         self.d_seq_lens = torch.zeros(self.Bmax, dtype=torch.int32, device=d)
+        # decode rows are one-token sequences: row r is sequence r
+        self.d_state_slots = torch.zeros(self.Bmax, dtype=torch.int32,
+                                         device=d)
+        self.d_row_seq = torch.arange(self.Bmax, dtype=torch.int32, device=d)
+        self.d_cu_rows = torch.arange(self.Bmax + 1, dtype=torch.int32,
+                                      device=d)
         self.d_temps = torch.zeros(self.Bmax, dtype=torch.float32, device=d)
         self.d_topk = torch.zeros(self.Bmax, dtype=torch.int32, device=d)
         self.d_topp = torch.ones(self.Bmax, dtype=torch.float32, device=d)
@@ -140,6 +180,8 @@ class LLMEngine:
                                   pin_memory=pin)
         self.h_seq_lens = torch.zeros(self.Bmax, dtype=torch.int32,
                                       pin_memory=pin)
+        self.h_state_slots = torch.zeros(self.Bmax, dtype=torch.int32,
+                                         pin_memory=pin)
         self.h_bt = torch.zeros(self.Bmax, mb, dtype=torch.int32,
                                 pin_memory=pin)
         self.h_params = torch.zeros(self.Bmax, 3, dtype=torch.float32,
@@ -152,6 +194,7 @@ class LLMEngine:
         self.n_pos = self.h_pos.numpy()
         self.n_slots = self.h_slots.numpy()
         self.n_seq_lens = self.h_seq_lens.numpy()
+        self.n_state_slots = self.h_state_slots.numpy()
         self.n_bt = self.h_bt.numpy()
 
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
@@ -179,10 +222,18 @@ class LLMEngine:
                                     ctx_start=kv.num_tokens))
         return rid
 
-    def free_sequence(self, kv: SequenceKV) -> None:
+    def _drop_cached(self, kv: SequenceKV) -> None:
+        """Give back a sequence's pages and its state slot; the sequence
+        restarts from position 0 when it runs again."""
         self.kv.allocator.free(kv.blocks)
         kv.blocks = []
         kv.num_tokens = 0
+        if self.states is not None and kv.state_slot >= 0:
+            self.states.free(kv.state_slot)
+        kv.state_slot = -1
+
+    def free_sequence(self, kv: SequenceKV) -> None:
+        self._drop_cached(kv)
         kv.pending_token = None
         kv.history = []
 
@@ -255,9 +306,7 @@ class LLMEngine:
             return False
         log.info("evicting idle session KV (%d blocks) to unblock admission",
                  len(victim.blocks))
-        self.kv.allocator.free(victim.blocks)
-        victim.blocks = []
-        victim.num_tokens = 0
+        self._drop_cached(victim)
         return True
 
     # ------------------------------------------------------------------
@@ -271,6 +320,7 @@ class LLMEngine:
         tokens = 0
         free = self.kv.allocator.num_free
         avail_rows = len(self._free_rows)
+        free_slots = self.states.num_free if self.states is not None else None
         budget = self.ecfg.max_prefill_tokens
         # soft tail: a request whose remainder only slightly overflows the
         # budget is admitted whole rather than leaving a tiny (<1/16
@@ -294,6 +344,11 @@ class LLMEngine:
             if need > free:
                 blocked = True
                 break
+            if free_slots is not None and req.kv.state_slot < 0:
+                if free_slots <= 0:
+                    blocked = True
+                    break
+                free_slots -= 1
             free -= need
             tokens += chunk
             if finishing:
@@ -305,25 +360,34 @@ class LLMEngine:
         return batch, blocked
 
     def _alloc_for(self, req: Request, new_tokens: int) -> List[int]:
-        need = req.kv.blocks_needed(new_tokens)
+        return self._alloc_tokens(req.kv, new_tokens)
+
+    def _alloc_tokens(self, kv: SequenceKV, new_tokens: int) -> List[int]:
+        need = kv.blocks_needed(new_tokens)
         if need:
-            req.kv.blocks.extend(self.kv.allocator.alloc(need))
-        slots = req.kv.slots_for(new_tokens)
-        req.kv.num_tokens += new_tokens
+            kv.blocks.extend(self.kv.allocator.alloc(need))
+        if self.states is not None and kv.state_slot < 0:
+            kv.state_slot = self.states.alloc()
+        slots = kv.slots_for(new_tokens)
+        kv.num_tokens += new_tokens
         return slots
 
     # ------------------------------------------------------------------
-    def _run_prefill(self, batch: List[Tuple[Request, int]]) -> List[StepOutput]:
+    def _packed_forward(self, items, mode: str = "prefill"):
+        """Run the next tokens of several sequences as ONE packed batch:
+        items = [(SequenceKV, tokens)]. Allocates pages (and a state slot)
+        for the new tokens, builds the attention metadata and calls the
+        model. -> hidden [sum(len(tokens)), W] (final-normed)."""
         dev = self.device
         ids, pos, slots = [], [], []
         qs_pairs, qb_seq, qb_start = [], [], []
+        row_seq, cu_rows = [], [0]
         row = 0
-        for s, (req, chunk) in enumerate(batch):
-            toks = req.prompt_tokens[req.prefill_pos:
-                                     req.prefill_pos + chunk]
-            start = req.kv.num_tokens
-            sl = self._alloc_for(req, chunk)
-            req.kv.history.extend(toks)
+        for s, (kv, toks) in enumerate(items):
+            chunk = len(toks)
+            start = kv.num_tokens
+            sl = self._alloc_tokens(kv, chunk)
+            kv.history.extend(toks)
             ids.extend(toks)
             pos.extend(range(start, start + chunk))
             slots.extend(sl)
@@ -331,27 +395,81 @@ class LLMEngine:
             for qb in range(0, chunk, 32):
                 qb_seq.append(s)
                 qb_start.append(qb)
+            row_seq.extend([s] * chunk)
             row += chunk
+            cu_rows.append(row)
+
+        def i32(x):
+            return torch.tensor(x, dtype=torch.int32, device=dev)
+
+        mbt = max(len(kv.blocks) for kv, _ in items)
+        bt = torch.zeros(len(items), mbt, dtype=torch.int32)
+        for i, (kv, _) in enumerate(items):
+            bt[i, : len(kv.blocks)] = torch.tensor(kv.blocks,
+                                                   dtype=torch.int32)
+        meta = AttnMeta(mode=mode, positions=i32(pos),
+                        slot_mapping=i32(slots),
+                        block_table=bt.to(dev),
+                        seq_lens=i32([kv.num_tokens for kv, _ in items]),
+                        q_starts=i32(qs_pairs), qb_seq=i32(qb_seq),
+                        qb_start=i32(qb_start))
+        if self.layered:
+            meta.row_seq = i32(row_seq)
+            meta.cu_rows = i32(cu_rows)
+            meta.state_slots = i32([max(kv.state_slot, 0)
+                                    for kv, _ in items])
+            meta.state = self.states.layers if self.states else None
+            meta.max_rows = max(len(t) for _, t in items)
+        return self.model.forward(i32(ids), self.kv.k, self.kv.v, meta)
+
+    def forward_tokens(self, entries, want=None) -> torch.Tensor:
+        """Teacher-forced step: feed given tokens instead of sampled ones.
+
+        entries = [(SequenceKV, tokens)] — each sequence's NEXT tokens, a
+        prompt portion or a single token, all run as one batch on top of
+        what the cache and state slots hold. `want[i]` lists the places in
+        entries[i]'s tokens whose logits are returned (default: the last).
+        -> fp32 logits [sum(len(want[i])), vocab], in entry order. A step
+        of single tokens only takes the decode kernels, anything else the
+        packed-portion kernels — the same ones generation runs."""
+        items = [(kv, list(toks)) for kv, toks in entries if len(toks)]
+        if not items:
+            return torch.empty(0, self.cfg.vocab_size, dtype=torch.float32,
+                               device=self.device)
+        for kv, toks in items:
+            self._known_kvs[id(kv)] = kv
+            if kv.num_tokens + len(toks) > self.ecfg.max_model_len:
+                raise ValueError("sequence exceeds max_model_len")
+        need = sum(kv.blocks_needed(len(t)) for kv, t in items)
+        if need > self.kv.allocator.num_free:
+            raise MemoryError(
+                f"KV cache exhausted: want {need} blocks, "
+                f"{self.kv.allocator.num_free} free")
+        decode = all(len(t) == 1 and kv.num_tokens > 0 for kv, t in items)
+        hidden = self._packed_forward(items,
+                                      "decode" if decode else "prefill")
+        rows, acc, j = [], 0, 0
+        for i, (kv, toks) in enumerate(entries):
+            if not len(toks):
+                continue
+            w = want[i] if want is not None else [len(toks) - 1]
+            rows.extend(acc + int(p) for p in w)
+            acc += len(toks)
+        if not rows:
+            return torch.empty(0, self.cfg.vocab_size, dtype=torch.float32,
+                               device=self.device)
+        sel = hidden[torch.tensor(rows, dtype=torch.long,
+                                  device=self.device)]
+        return self.model.compute_logits(sel).float()
+
+    def _run_prefill(self, batch: List[Tuple[Request, int]]) -> List[StepOutput]:
+        dev = self.device
+        items = []
+        for req, chunk in batch:
+            items.append((req.kv, req.prompt_tokens[
+                req.prefill_pos: req.prefill_pos + chunk]))
             req.prefill_pos += chunk
-        t_ids = torch.tensor(ids, dtype=torch.int32, device=dev)
-        t_pos = torch.tensor(pos, dtype=torch.int32, device=dev)
-        t_slots = torch.tensor(slots, dtype=torch.int32, device=dev)
-        t_seq_lens = torch.tensor([r.kv.num_tokens for r, _ in batch],
-                                  dtype=torch.int32, device=dev)
-        t_qs = torch.tensor(qs_pairs, dtype=torch.int32, device=dev)
-        mbt = max(len(r.kv.blocks) for r, _ in batch)
-        bt = torch.zeros(len(batch), mbt, dtype=torch.int32)
-        for i, (r, _) in enumerate(batch):
-            bt[i, : len(r.kv.blocks)] = torch.tensor(r.kv.blocks,
-                                                     dtype=torch.int32)
-        meta = AttnMeta(mode="prefill", positions=t_pos, slot_mapping=t_slots,
-                        block_table=bt.to(dev), seq_lens=t_seq_lens,
-                        q_starts=t_qs,
-                        qb_seq=torch.tensor(qb_seq, dtype=torch.int32,
-                                            device=dev),
-                        qb_start=torch.tensor(qb_start, dtype=torch.int32,
-                                              device=dev))
-        hidden = self.model.forward(t_ids, self.kv.k, self.kv.v, meta)
+        hidden = self._packed_forward(items)
         # sample only the requests whose prompt completed this pass
         finishing = [(i, r) for i, (r, _) in enumerate(batch)
                      if r.prefill_pos == len(r.prompt_tokens)]
@@ -378,6 +496,8 @@ class LLMEngine:
         tp = torch.tensor([r.sampling.top_p for r in reqs],
                           dtype=torch.float32, device=dev)
         tokens = torch.zeros(B, dtype=torch.int32, device=dev)
+        if logits.dtype != torch.bfloat16:
+            logits = logits.to(torch.bfloat16)
         ops.sample(tokens, logits.contiguous(), temps, tk, tp, self.d_seed,
                    self.d_ws[:B])
         return tokens.cpu().tolist()
@@ -474,9 +594,7 @@ class LLMEngine:
         self._release_row(req)
         history = list(req.kv.history)
         last = req.output_tokens[-1] if req.output_tokens else None
-        self.kv.allocator.free(req.kv.blocks)
-        req.kv.blocks = []
-        req.kv.num_tokens = 0
+        self._drop_cached(req.kv)
         req.kv.history = []
         req.kv.pending_token = None
         req.prompt_tokens = history + ([last] if last is not None else [])
@@ -526,6 +644,7 @@ class LLMEngine:
             self.n_ids[row] = r.output_tokens[-1]
             self.n_pos[row] = start
             self.n_seq_lens[row] = start + 1
+            self.n_state_slots[row] = max(r.kv.state_slot, 0)
             n = len(r.kv.blocks)
             if n > r.bt_written:
                 self.n_bt[row, r.bt_written: n] = r.kv.blocks[r.bt_written:]
@@ -543,6 +662,9 @@ class LLMEngine:
         self.d_pos[:nb].copy_(self.h_pos[:nb], non_blocking=True)
         self.d_seq_lens[:nb].copy_(self.h_seq_lens[:nb], non_blocking=True)
         self.d_bt[:nb].copy_(self.h_bt[:nb], non_blocking=True)
+        if self.states is not None:
+            self.d_state_slots[:nb].copy_(self.h_state_slots[:nb],
+                                          non_blocking=True)
         if self._params_dirty:
             self.d_temps.copy_(self.h_params[:, 0], non_blocking=True)
             self.d_topk.copy_(self.h_params[:, 1].to(torch.int32),
@@ -591,15 +713,28 @@ class LLMEngine:
         return outs
 
     def _decode_forward(self, B: int) -> None:
-        splits = self._decode_splits(B)
-        tmp_out, tmp_ml = self._tmp_for(B, splits)
-        meta = AttnMeta(
-            mode="decode", positions=self.d_pos[:B],
-            slot_mapping=self.d_slots[:B], block_table=self.d_bt[:B],
-            seq_lens=self.d_seq_lens[:B], num_splits=splits,
-            tmp_out=tmp_out, tmp_ml=tmp_ml)
+        if self.layered:
+            meta = AttnMeta(
+                mode="decode", positions=self.d_pos[:B],
+                slot_mapping=self.d_slots[:B], block_table=self.d_bt[:B],
+                seq_lens=self.d_seq_lens[:B])
+            meta.row_seq = self.d_row_seq[:B]
+            meta.cu_rows = self.d_cu_rows[:B + 1]
+            meta.state_slots = self.d_state_slots[:B]
+            meta.state = self.states.layers if self.states else None
+            meta.max_rows = 1
+        else:
+            splits = self._decode_splits(B)
+            tmp_out, tmp_ml = self._tmp_for(B, splits)
+            meta = AttnMeta(
+                mode="decode", positions=self.d_pos[:B],
+                slot_mapping=self.d_slots[:B], block_table=self.d_bt[:B],
+                seq_lens=self.d_seq_lens[:B], num_splits=splits,
+                tmp_out=tmp_out, tmp_ml=tmp_ml)
         hidden = self.model.forward(self.d_ids[:B], self.kv.k, self.kv.v, meta)
         logits = self.model.compute_logits(hidden)
+        if logits.dtype != torch.bfloat16:
+            logits = logits.to(torch.bfloat16)
         ops.sample(self.d_tokens[:B], logits, self.d_temps[:B],
                    self.d_topk[:B], self.d_topp[:B], self.d_seed,
                    self.d_ws[:B])

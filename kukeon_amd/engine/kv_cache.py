@@ -9,7 +9,8 @@ sized for 288 GB HBM").
 """
 from __future__ import annotations
 
-from typing import List
+from dataclasses import dataclass
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -47,6 +48,8 @@ class SequenceKV:
         # last sampled token of the previous turn: sampled but never run
         # through the model, so the next turn's prefill must include it
         self.pending_token = None
+        # slot of this sequence in the engine's StatePool (-1: none held)
+        self.state_slot = -1
         # every token whose K/V lives in the cache, in order — the replay
         # source for preemption-by-recompute
         self.history = []
@@ -88,3 +91,101 @@ class PagedKVCache:
                           dtype_bytes: int = 2) -> int:
         per_block = 2 * num_layers * num_kv_heads * block_size * head_dim * dtype_bytes
         return max(1, free_bytes // per_block)
+
+
+@dataclass
+class LayerKVSpec:
+    """Cache geometry of one layer. A layer with `share_from` set keeps no
+    pages of its own: it reads the pages of that (earlier) layer."""
+    kv_heads: int
+    k_width: int
+    v_width: int
+    share_from: Optional[int] = None
+
+
+class LayeredKVCache:
+    """Paged cache whose layers differ in shape (key rows wider than value
+    rows, per-layer head counts) and may share pages across layers.
+
+    One allocator serves all layers: block id b names the page
+    [b, kv_heads, block_size, width] in every layer's pool, so a sequence
+    holds ONE block list. `k[i]` / `v[i]` of a sharing layer alias the
+    owner's tensors.
+    """
+
+    def __init__(self, specs: Sequence[LayerKVSpec], num_blocks: int,
+                 block_size: int, device, dtype=torch.bfloat16):
+        self.specs = list(specs)
+        self.num_layers = len(self.specs)
+        self.num_blocks = num_blocks
+        self.block_size = block_size
+        self.k: List[torch.Tensor] = [None] * self.num_layers
+        self.v: List[torch.Tensor] = [None] * self.num_layers
+        for i, sp in enumerate(self.specs):
+            if sp.share_from is not None:
+                continue
+            # zeros: masked-out tail slots are never read as garbage
+            self.k[i] = torch.zeros(num_blocks, sp.kv_heads, block_size,
+                                    sp.k_width, dtype=dtype, device=device)
+            self.v[i] = torch.zeros(num_blocks, sp.kv_heads, block_size,
+                                    sp.v_width, dtype=dtype, device=device)
+        for i, sp in enumerate(self.specs):
+            if sp.share_from is None:
+                continue
+            j = sp.share_from
+            if not (0 <= j < i) or self.specs[j].share_from is not None:
+                raise ValueError(
+                    f"layer {i} shares the cache of layer {j}, which must be "
+                    "an earlier layer with pages of its own")
+            own = self.specs[j]
+            if (own.kv_heads, own.k_width, own.v_width) != \
+                    (sp.kv_heads, sp.k_width, sp.v_width):
+                raise ValueError(
+                    f"layer {i} and the layer {j} it shares with differ in "
+                    "cache shape")
+            self.k[i], self.v[i] = self.k[j], self.v[j]
+        self.allocator = BlockAllocator(num_blocks)
+
+    @property
+    def nbytes(self) -> int:
+        return sum(self.k[i].nbytes + self.v[i].nbytes
+                   for i, sp in enumerate(self.specs)
+                   if sp.share_from is None)
+
+    @staticmethod
+    def blocks_from_bytes(free_bytes: int, specs: Sequence[LayerKVSpec],
+                          block_size: int, dtype_bytes: int = 2) -> int:
+        per_block = sum(sp.kv_heads * block_size * (sp.k_width + sp.v_width)
+                        for sp in specs if sp.share_from is None) * dtype_bytes
+        return max(1, free_bytes // max(1, per_block))
+
+
+class StatePool:
+    """Fixed-size slots of per-sequence carried state (tails of short
+    convolutions, recurrent state): one fp32 tensor [slots, *shape] per
+    layer that carries state, None for the others. A sequence holds one
+    slot index for all layers; a slot's content is only meaningful to the
+    sequence that wrote it, and a sequence that starts at position 0 never
+    reads what the slot held before."""
+
+    def __init__(self, layer_shapes: Sequence[Optional[Tuple[int, ...]]],
+                 num_slots: int, device, dtype=torch.float32):
+        self.num_slots = num_slots
+        self.layers: List[Optional[torch.Tensor]] = [
+            None if shp is None else
+            torch.zeros((num_slots,) + tuple(shp), dtype=dtype, device=device)
+            for shp in layer_shapes]
+        self._free: List[int] = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def alloc(self) -> int:
+        if not self._free:
+            raise MemoryError("state slots exhausted")
+        return self._free.pop()
+
+    def free(self, slot: int) -> None:
+        if slot >= 0:
+            self._free.append(slot)

@@ -35,6 +35,14 @@ class AttnMeta:
     num_splits: int = 1
     tmp_out: Optional[torch.Tensor] = None    # decode split-KV workspaces
     tmp_ml: Optional[torch.Tensor] = None
+    # packed-row maps and carried state, for models whose kernels take
+    # them (row r belongs to sequence row_seq[r]; sequence s owns rows
+    # cu_rows[s] .. cu_rows[s+1]-1 and state slot state_slots[s])
+    row_seq: Optional[torch.Tensor] = None    # [T] int32
+    cu_rows: Optional[torch.Tensor] = None    # [nseq+1] int32
+    state_slots: Optional[torch.Tensor] = None  # [nseq] int32
+    state: Optional[list] = None              # per-layer state tensors
+    max_rows: int = 0                         # longest portion in the batch
 
 
 def split_prefill_meta(meta: AttnMeta, parts: int = 2):

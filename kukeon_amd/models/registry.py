@@ -1,0 +1,74 @@
+"""Model registry: which class serves which architecture.
+
+Built-in presets (random-init benchmark shapes) are looked up by name; a
+checkpoint folder is dispatched on the `architecture` field of its
+config.json."""
+from __future__ import annotations
+
+import json
+import os
+from typing import Callable, Dict
+
+from kukeon_amd.engine.config import MODEL_PRESETS
+
+
+def _llama(cfg, device, **kw):
+    from kukeon_amd.models.llama import LlamaModel
+    return LlamaModel(cfg, device=device)
+
+
+def _mixtral(cfg, device, **kw):
+    from kukeon_amd.models.mixtral import MixtralModel
+    return MixtralModel(cfg, device=device)
+
+
+def _lipedra(cfg, device, **kw):
+    from kukeon_amd.models.lipedra import LipedraModel
+    return LipedraModel(cfg, device=device, **kw)
+
+
+# family -> constructor(cfg, device, **kw)
+FAMILIES: Dict[str, Callable] = {
+    "llama": _llama,
+    "mixtral": _mixtral,
+    "lipedra": _lipedra,
+}
+
+# config.json "architecture" -> family
+ARCHITECTURES: Dict[str, str] = {
+    "Lipedra": "lipedra",
+}
+
+
+def family_of(cfg) -> str:
+    fam = getattr(cfg, "family", None)
+    if fam:
+        return fam
+    return "mixtral" if getattr(cfg, "is_moe", False) else "llama"
+
+
+def build_model(cfg, device, **kw):
+    """Instantiate (random-init) the model class that serves `cfg`."""
+    return FAMILIES[family_of(cfg)](cfg, device, **kw)
+
+
+def preset(name: str):
+    if name not in MODEL_PRESETS:
+        raise KeyError(f"unknown model preset {name!r}; known: "
+                       f"{sorted(MODEL_PRESETS)}")
+    return MODEL_PRESETS[name]()
+
+
+def load_checkpoint(model_dir: str, device, dtype: str = "bf16"):
+    """-> (cfg, model) for a folder with config.json + model.safetensors."""
+    with open(os.path.join(model_dir, "config.json")) as f:
+        arch = json.load(f).get("architecture")
+    fam = ARCHITECTURES.get(arch)
+    if fam is None:
+        raise ValueError(f"no model class registered for architecture "
+                         f"{arch!r}; known: {sorted(ARCHITECTURES)}")
+    if fam == "lipedra":
+        from kukeon_amd.models.lipedra import LipedraModel
+        return LipedraModel.from_checkpoint(model_dir, device=device,
+                                            dtype=dtype)
+    raise ValueError(f"family {fam} has no checkpoint loader")

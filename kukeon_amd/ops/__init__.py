@@ -19,8 +19,33 @@ except Exception as e:  # pragma: no cover - exercised only on broken installs
     _IMPORT_ERROR = e
 
 
+_C_mix = None
+_MIX_IMPORT_ERROR: Exception | None = None
+try:
+    from kukeon_amd import _C_mix  # type: ignore
+except Exception as e:  # pragma: no cover
+    _MIX_IMPORT_ERROR = e
+
+
 def native_available() -> bool:
     return _C is not None
+
+
+def mix_available() -> bool:
+    return _C_mix is not None
+
+
+def _mix(t: torch.Tensor):
+    """Kernel group of the sequence mixers: native on a GPU tensor (an
+    error if the module is not built), the fp32 references on CPU."""
+    if not t.is_cuda:
+        return reference
+    if _C_mix is None:
+        raise RuntimeError(
+            "kukeon_amd._C_mix (gfx950 HIP extension) is not built but an op "
+            "was called on a CUDA device. Run `python -m kukeon_amd.ops.build "
+            f"mix` (import error: {_MIX_IMPORT_ERROR})")
+    return _C_mix
 
 
 def _native():
@@ -280,3 +305,54 @@ def moe_gather_tokens(out, input, row_map) -> None:
 
 def moe_scatter_tokens(out, input, inv_map, weights, top_k: int) -> None:
     _impl(input).moe_scatter_tokens(out, input, inv_map, weights, top_k)
+
+
+# ---- sequence-mixer group -------------------------------------------------
+def _e(t: torch.Tensor):
+    return torch.empty(0, dtype=t.dtype, device=t.device)
+
+
+def residual_add_rmsnorm(x, a, bias, w, w_offset: float, eps: float,
+                         out) -> None:
+    """x (fp32 residual, in place) += a (+ bias); out = rmsnorm(x) scaled by
+    (w_offset + w). `a` / `bias` may be None."""
+    _mix(x).residual_add_rmsnorm(
+        x, a if a is not None else _e(out),
+        bias if bias is not None else _e(x), w, w_offset, eps, out)
+
+
+def clamp_glu(out, gate, up, bg, bu, limit: float, alpha: float = 1.702,
+              up_shift: float = 1.0) -> None:
+    _mix(out).clamp_glu(out, gate, up,
+                        bg if bg is not None else _e(bu if bu is not None
+                                                     else out.float()),
+                        bu if bu is not None else _e(out.float()),
+                        limit, alpha, up_shift)
+
+
+def conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw, state, cs,
+                     positions, row_seq, cu_rows, state_slots, block_table,
+                     q_col: int, k_col: int, v_col: int, Cq: int, Ck: int,
+                     Cv: int, map_dim: int, rot_dims: int) -> None:
+    if k_cache is None:
+        k_cache = v_cache = _e(proj)
+    _mix(proj).conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw,
+                                state, cs, positions, row_seq, cu_rows,
+                                state_slots, block_table, q_col, k_col, v_col,
+                                Cq, Ck, Cv, map_dim, rot_dims)
+
+
+def conv_state_update(state, proj, bias, positions, cu_rows, state_slots,
+                      q_col: int, k_col: int, v_col: int, Cq: int, Ck: int,
+                      Cv: int) -> None:
+    _mix(proj).conv_state_update(state, proj, bias, positions, cu_rows,
+                                 state_slots, q_col, k_col, v_col, Cq, Ck, Cv)
+
+
+def diff_attention(out, q, k_cache, v_cache, gate, positions, row_seq,
+                   block_table, H: int, scale: float, lam: float, eps: float,
+                   out_scale: float) -> None:
+    _mix(q).diff_attention(out, q, k_cache, v_cache,
+                           gate if gate is not None else _e(q), positions,
+                           row_seq, block_table, H, scale, lam, eps,
+                           out_scale)

@@ -18,6 +18,19 @@ OBJ_DIR = PKG_DIR / "ops" / "_build"
 SO_PATH = PKG_DIR / "_C.so"
 ARCH = os.environ.get("KUKEON_GFX_ARCH", "gfx950")
 
+# Kernel groups: each links into its own module, so a model that needs one
+# group does not wait for the others to compile.
+#   core -> kukeon_amd/_C.so      (Llama/Mixtral op set, sampler, GEMMs)
+#   mix  -> kukeon_amd/_C_mix.so  (fp32-residual norm, clamped GLU, short
+#                                  convolution + rotary, differential attention)
+MIX_SOURCES = [
+    "resid_norm.hip",
+    "glu_clamp.hip",
+    "short_conv.hip",
+    "diff_attn.hip",
+    "bindings_mix.cpp",
+]
+
 SOURCES = [
     "rmsnorm.hip",
     "activation.hip",
@@ -45,7 +58,28 @@ def _run(cmd: list[str]) -> None:
         raise RuntimeError(f"build command failed (rc={proc.returncode})")
 
 
-def build(verbose: bool = True, force: bool = False) -> Path:
+GROUPS = {
+    "core": ("_C", SOURCES),
+    "mix": ("_C_mix", MIX_SOURCES),
+}
+
+
+def so_path(group: str) -> Path:
+    return PKG_DIR / (GROUPS[group][0] + ".so")
+
+
+def build(verbose: bool = True, force: bool = False,
+          groups=None) -> Path:
+    """Compile and link the given kernel groups (default: all)."""
+    out = None
+    for g in (groups or list(GROUPS)):
+        out = _build_group(g, verbose, force)
+    return out
+
+
+def _build_group(group: str, verbose: bool, force: bool) -> Path:
+    modname, sources = GROUPS[group]
+    SO_PATH = so_path(group)
     inc, libdirs = _torch_paths()
     py_inc = sysconfig.get_paths()["include"]
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
@@ -58,7 +92,9 @@ def build(verbose: bool = True, force: bool = False) -> Path:
         "-DNDEBUG",
         "-D__HIP_NO_HALF_OPERATORS__=1",
         "-D__HIP_NO_HALF_CONVERSIONS__=1",
-        "-DTORCH_EXTENSION_NAME=_C",
+        f"-DTORCH_EXTENSION_NAME={modname}",
+        # packed fp32 VALU forms are kept out of all device code
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         "-DUSE_ROCM=1",
         "-DTORCH_API_INCLUDE_EXTENSION_H",
         "-D_GLIBCXX_USE_CXX11_ABI=1",
@@ -70,20 +106,31 @@ def build(verbose: bool = True, force: bool = False) -> Path:
 
     hdr_mtime = max(p.stat().st_mtime for p in CSRC.glob("*.h"))
     objs = []
-    for src in SOURCES:
+    todo = []
+    for src in sources:
         sp = CSRC / src
         op = OBJ_DIR / (src.rsplit(".", 1)[0] + ".o")
         objs.append(op)
         if (not force and op.exists()
                 and op.stat().st_mtime > max(sp.stat().st_mtime, hdr_mtime)):
             continue
-        if verbose:
-            print(f"[kukeon_amd.build] hipcc -c {src}")
         cmd = ["hipcc", "-c", str(sp), "-o", str(op)] + common_flags
         if src.endswith(".cpp"):
             cmd.append("-x")
             cmd.append("c++")
-        _run(cmd)
+        todo.append((src, cmd))
+
+    def _one(item):
+        if verbose:
+            print(f"[kukeon_amd.build] hipcc -c {item[0]}", flush=True)
+        _run(item[1])
+
+    if todo:
+        from concurrent.futures import ThreadPoolExecutor
+        jobs = max(1, min(len(todo), int(os.environ.get("MAX_JOBS", "0") or 0)
+                          or (os.cpu_count() or 4), 16))
+        with ThreadPoolExecutor(jobs) as pool:
+            list(pool.map(_one, todo))
 
     if force or not SO_PATH.exists() or any(
             o.stat().st_mtime > SO_PATH.stat().st_mtime for o in objs):
@@ -104,5 +151,7 @@ def build(verbose: bool = True, force: bool = False) -> Path:
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv)
-    print(f"built {SO_PATH}")
+    names = [a for a in sys.argv[1:] if not a.startswith("-")]
+    build(force="--force" in sys.argv, groups=names or None)
+    for g in (names or list(GROUPS)):
+        print(f"built {so_path(g)}")

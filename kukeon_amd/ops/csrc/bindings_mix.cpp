@@ -1,0 +1,46 @@
+// Python bindings for the sequence-mixer kernel group (fp32 residual norm,
+// clamped gated activation, short convolution + rotary + KV append,
+// differential attention). Built as its own module so a model that needs
+// only these does not wait for the rest of the kernel library.
+#include <torch/extension.h>
+
+namespace kukeon {
+void residual_add_rmsnorm(torch::Tensor x, torch::Tensor a, torch::Tensor bias,
+                          torch::Tensor w, double w_offset, double eps,
+                          torch::Tensor out);
+void clamp_glu(torch::Tensor out, torch::Tensor gate, torch::Tensor up,
+               torch::Tensor bg, torch::Tensor bu, double limit, double alpha,
+               double up_shift);
+void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
+                      torch::Tensor v_cache, torch::Tensor proj,
+                      torch::Tensor bias, torch::Tensor cw,
+                      torch::Tensor state, torch::Tensor cs,
+                      torch::Tensor positions, torch::Tensor row_seq,
+                      torch::Tensor cu_rows, torch::Tensor state_slots,
+                      torch::Tensor block_table, int64_t q_col, int64_t k_col,
+                      int64_t v_col, int64_t Cq, int64_t Ck, int64_t Cv,
+                      int64_t map_dim, int64_t rot_dims);
+void conv_state_update(torch::Tensor state, torch::Tensor proj,
+                       torch::Tensor bias, torch::Tensor positions,
+                       torch::Tensor cu_rows, torch::Tensor state_slots,
+                       int64_t q_col, int64_t k_col, int64_t v_col, int64_t Cq,
+                       int64_t Ck, int64_t Cv);
+void diff_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
+                    torch::Tensor v_cache, torch::Tensor gate,
+                    torch::Tensor positions, torch::Tensor row_seq,
+                    torch::Tensor block_table, int64_t H, double scale,
+                    double lambda, double eps, double out_scale);
+}  // namespace kukeon
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("residual_add_rmsnorm", &kukeon::residual_add_rmsnorm,
+        "fp32 residual += a (+bias); out = rmsnorm(x) * (offset + w)");
+  m.def("clamp_glu", &kukeon::clamp_glu,
+        "clamped gate * sigmoid(alpha gate) * (up + shift)");
+  m.def("conv_rope_append", &kukeon::conv_rope_append,
+        "bias + short causal conv (carried state) + rotary + paged KV append");
+  m.def("conv_state_update", &kukeon::conv_state_update,
+        "shift a portion's tail into the convolution state slots");
+  m.def("diff_attention", &kukeon::diff_attention,
+        "paged differential attention with unit norm and output gate");
+}

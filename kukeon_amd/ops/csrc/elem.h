@@ -1,0 +1,85 @@
+// Element access for kernels that serve two activation formats: bf16
+// (stored as raw ushort) for serving and float for the exact mode. All
+// arithmetic is fp32 either way; only loads and stores differ.
+#pragma once
+#include "common.h"
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+
+namespace kukeon {
+
+typedef unsigned short bf16_t;
+
+DEV_INLINE float ldf(const float* p) { return *p; }
+DEV_INLINE float ldf(const bf16_t* p) { return us2f(*p); }
+DEV_INLINE void stf(float* p, float v) { *p = v; }
+DEV_INLINE void stf(bf16_t* p, float v) { *p = f2us(v); }
+
+// both-sum block reduction of a pair (one pass of barriers for two values)
+DEV_INLINE float2 block_sum2(float a, float b, float* red /* >= 32 floats */) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wid = threadIdx.x / WAVE;
+  const int nwaves = (blockDim.x + WAVE - 1) / WAVE;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    a += __shfl_xor(a, off, WAVE);
+    b += __shfl_xor(b, off, WAVE);
+  }
+  if (lane == 0) { red[2 * wid] = a; red[2 * wid + 1] = b; }
+  __syncthreads();
+  float ra = 0.f, rb = 0.f;
+  for (int w = 0; w < nwaves; ++w) { ra += red[2 * w]; rb += red[2 * w + 1]; }
+  __syncthreads();
+  return float2{ra, rb};
+}
+DEV_INLINE float2 block_max2(float a, float b, float* red) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wid = threadIdx.x / WAVE;
+  const int nwaves = (blockDim.x + WAVE - 1) / WAVE;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    a = fmaxf(a, __shfl_xor(a, off, WAVE));
+    b = fmaxf(b, __shfl_xor(b, off, WAVE));
+  }
+  if (lane == 0) { red[2 * wid] = a; red[2 * wid + 1] = b; }
+  __syncthreads();
+  float ra = -INFINITY, rb = -INFINITY;
+  for (int w = 0; w < nwaves; ++w) {
+    ra = fmaxf(ra, red[2 * w]);
+    rb = fmaxf(rb, red[2 * w + 1]);
+  }
+  __syncthreads();
+  return float2{ra, rb};
+}
+
+inline bool is_bf16(const torch::Tensor& t) {
+  return t.scalar_type() == torch::kBFloat16;
+}
+inline void check_act(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda(), name, " must be a device tensor");
+  TORCH_CHECK(t.scalar_type() == torch::kBFloat16 ||
+                  t.scalar_type() == torch::kFloat32,
+              name, " must be bf16 or fp32");
+}
+inline void check_f32(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat32 &&
+                  t.is_contiguous(), name, " must be contiguous fp32");
+}
+inline void check_i32(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kInt32 &&
+                  t.is_contiguous(), name, " must be contiguous int32");
+}
+
+// run BODY with `T` bound to the storage type of tensor `t`
+#define KK_DISPATCH_ACT(t, ...)             \
+  do {                                      \
+    if (is_bf16(t)) {                       \
+      typedef bf16_t T;                     \
+      __VA_ARGS__                           \
+    } else {                                \
+      typedef float T;                      \
+      __VA_ARGS__                           \
+    }                                       \
+  } while (0)
+
+}  // namespace kukeon

@@ -1,0 +1,64 @@
+// Clamped gated activation for a fused [.. gate .. up ..] projection row:
+//   g = min(gate + bg, limit), u = clamp(up + bu, -limit, limit)
+//   y = g * sigmoid(alpha * g) * (u + up_shift)
+// The projection biases are added here (in fp32) instead of in the GEMM.
+#include "elem.h"
+
+namespace kukeon {
+
+template <typename T>
+__global__ __launch_bounds__(256) void clamp_glu_kernel(
+    T* __restrict__ out, long ldo, const T* __restrict__ gate,
+    const T* __restrict__ up, long ldg, const float* __restrict__ bg,
+    const float* __restrict__ bu, float limit, float alpha, float up_shift,
+    int F, long total) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long r = idx / F;
+  const int f = (int)(idx - r * F);
+  float g = ldf(gate + r * ldg + f) + (bg ? bg[f] : 0.f);
+  float u = ldf(up + r * ldg + f) + (bu ? bu[f] : 0.f);
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  const float sg = 1.0f / (1.0f + expf(-alpha * g));
+  stf(out + r * ldo + f, g * sg * (u + up_shift));
+}
+
+// out [T,F] view (stride(1)==1); gate, up [T,F] views into one projection
+// buffer sharing a row stride; bg, bu [F] fp32 or empty.
+void clamp_glu(torch::Tensor out, torch::Tensor gate, torch::Tensor up,
+               torch::Tensor bg, torch::Tensor bu, double limit, double alpha,
+               double up_shift) {
+  check_act(out, "out");
+  TORCH_CHECK(gate.scalar_type() == out.scalar_type() &&
+              up.scalar_type() == out.scalar_type());
+  TORCH_CHECK(out.dim() == 2 && gate.dim() == 2 && up.dim() == 2);
+  const long rows = out.size(0);
+  const int F = (int)out.size(1);
+  TORCH_CHECK(gate.size(0) == rows && up.size(0) == rows &&
+              gate.size(1) == F && up.size(1) == F);
+  TORCH_CHECK(out.stride(1) == 1 && gate.stride(1) == 1 &&
+              up.stride(1) == 1 && gate.stride(0) == up.stride(0));
+  const bool hb = bg.numel() > 0;
+  if (hb) {
+    check_f32(bg, "bg");
+    check_f32(bu, "bu");
+    TORCH_CHECK(bg.numel() == F && bu.numel() == F);
+  }
+  const long total = rows * F;
+  if (total == 0) return;
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+  KK_DISPATCH_ACT(out, {
+    clamp_glu_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0,
+                          stream>>>(
+        reinterpret_cast<T*>(out.data_ptr()), out.stride(0),
+        reinterpret_cast<const T*>(gate.data_ptr()),
+        reinterpret_cast<const T*>(up.data_ptr()), gate.stride(0),
+        hb ? bg.data_ptr<float>() : nullptr,
+        hb ? bu.data_ptr<float>() : nullptr, (float)limit, (float)alpha,
+        (float)up_shift, F, total);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+}  // namespace kukeon

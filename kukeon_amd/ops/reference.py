@@ -248,3 +248,138 @@ def moe_dense_combine(out: torch.Tensor, y: torch.Tensor,
                       wdense: torch.Tensor) -> None:
     acc = (y.float() * wdense.t().unsqueeze(-1)).sum(dim=0)
     out.copy_(acc.to(out.dtype))
+
+
+# ---------------------------------------------------------------------------
+# sequence-mixer group (fp32 residual stream; activations bf16 or fp32)
+# ---------------------------------------------------------------------------
+
+def residual_add_rmsnorm(x: torch.Tensor, a, bias, w: torch.Tensor,
+                         w_offset: float, eps: float,
+                         out: torch.Tensor) -> None:
+    """x (fp32, in place) += a (+ bias); out = x / rms(x) * (w_offset + w)."""
+    W = x.shape[1]
+    if a is not None and a.numel():
+        x += a[:, :W].float()
+    if bias is not None and bias.numel():
+        x += bias
+    rs = 1.0 / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    out.copy_((x * rs * (w_offset + w)).to(out.dtype))
+
+
+def clamp_glu(out, gate, up, bg, bu, limit: float, alpha: float,
+              up_shift: float) -> None:
+    g = gate.float()
+    u = up.float()
+    if bg is not None and bg.numel():
+        g = g + bg
+        u = u + bu
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    out.copy_((g * torch.sigmoid(alpha * g) * (u + up_shift)).to(out.dtype))
+
+
+def _conv_cols(q_col, k_col, v_col, Cq, Ck, Cv):
+    cols = list(range(q_col, q_col + Cq))
+    cols += list(range(k_col, k_col + Ck))
+    cols += list(range(v_col, v_col + Cv))
+    return torch.tensor(cols, dtype=torch.long)
+
+
+def conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw, state, cs,
+                     positions, row_seq, cu_rows, state_slots, block_table,
+                     q_col: int, k_col: int, v_col: int, Cq: int, Ck: int,
+                     Cv: int, map_dim: int, rot_dims: int) -> None:
+    C = Cq + Ck + Cv
+    taps = cw.shape[1]
+    back = taps - 1
+    cols = _conv_cols(q_col, k_col, v_col, Cq, Ck, Cv)
+    nseq = cu_rows.numel() - 1
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0 or int(positions[r0]) < 0:
+            continue
+        n = r1 - r0
+        p0 = int(positions[r0])
+        u = proj[r0:r1][:, cols].float() + bias              # [n, C]
+        hist = state[int(state_slots[s])].clone() if back else u[:0]
+        if back:
+            # entries that lie before the sequence start count as zeros
+            for k in range(back):
+                if p0 - back + k < 0:
+                    hist[k] = 0
+        full = torch.cat([hist, u], 0)                       # [back+n, C]
+        y = torch.zeros(n, C)
+        for j in range(taps):
+            y = y + cw[:, j] * full[j: j + n]
+        pos = positions[r0:r1].long()
+        ang = cs[pos.clamp(max=cs.shape[0] - 1)]             # [n, rot_dims]
+        half = rot_dims // 2
+        co, si = ang[:, :half], ang[:, half:]
+
+        def rot(seg):                                        # [n, maps*dim]
+            m = seg.reshape(n, -1, map_dim).clone()
+            a, b = m[..., 0:rot_dims:2], m[..., 1:rot_dims:2]
+            ra = a * co[:, None] - b * si[:, None]
+            rb = b * co[:, None] + a * si[:, None]
+            m[..., 0:rot_dims:2] = ra
+            m[..., 1:rot_dims:2] = rb
+            return m.reshape(n, -1)
+
+        q_out[r0:r1] = rot(y[:, :Cq]).to(q_out.dtype)
+        if Ck or Cv:
+            G, BS = k_cache.shape[1], k_cache.shape[2]
+            kk = rot(y[:, Cq:Cq + Ck]).reshape(n, G, -1).to(k_cache.dtype)
+            vv = y[:, Cq + Ck:].reshape(n, G, -1).to(v_cache.dtype)
+            for i in range(n):
+                p = p0 + i
+                blk = int(block_table[s, p // BS])
+                k_cache[blk, :, p % BS] = kk[i]
+                v_cache[blk, :, p % BS] = vv[i]
+
+
+def conv_state_update(state, proj, bias, positions, cu_rows, state_slots,
+                      q_col: int, k_col: int, v_col: int, Cq: int, Ck: int,
+                      Cv: int) -> None:
+    back = state.shape[1]
+    if back == 0:
+        return
+    cols = _conv_cols(q_col, k_col, v_col, Cq, Ck, Cv)
+    nseq = cu_rows.numel() - 1
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0 or int(positions[r0]) < 0:
+            continue
+        u = proj[r0:r1][:, cols].float() + bias
+        slot = int(state_slots[s])
+        full = torch.cat([state[slot], u], 0)
+        state[slot] = full[-back:]
+
+
+def diff_attention(out, q, k_cache, v_cache, gate, positions, row_seq,
+                   block_table, H: int, scale: float, lam: float, eps: float,
+                   out_scale: float) -> None:
+    G, BS = k_cache.shape[1], k_cache.shape[2]
+    dim = k_cache.shape[3] // 2
+    vdim = v_cache.shape[3]
+    rows = q.shape[0]
+    for r in range(rows):
+        p = int(positions[r])
+        if p < 0:
+            out[r, : H * vdim] = 0
+            continue
+        s = int(row_seq[r])
+        k = _gather_kv(k_cache, block_table, p + 1, s).float()  # [ctx,G,2d]
+        v = _gather_kv(v_cache, block_table, p + 1, s).float()
+        qr = q[r].float().view(H, 2, dim)
+        for h in range(H):
+            g = h // (H // G)
+            a = []
+            for m in range(2):
+                sc = (k[:, g, m * dim:(m + 1) * dim] @ qr[h, m]) * scale
+                a.append(torch.softmax(sc, -1) @ v[:, g])
+            o = a[0] - lam * a[1]
+            o = o / torch.sqrt(o.pow(2).mean() + eps) * out_scale
+            if gate is not None and gate.numel():
+                o = o * torch.sigmoid(gate[r, h].float())
+            out[r, h * vdim:(h + 1) * vdim] = o.to(out.dtype)
