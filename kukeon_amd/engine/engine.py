@@ -610,6 +610,12 @@ class LLMEngine:
         k = min(min(r.sampling.max_new_tokens - len(r.output_tokens)
                     for r in active0),
                 max(1, self.ecfg.decode_microbatch), self.max_microbatch)
+        if self.states is not None and any(r.sampling.stop_token_ids
+                                           for r in active0):
+            # a stop token inside a micro-batch leaves the device some
+            # steps ahead; pages can be rolled back by count, carried
+            # state cannot — step singly when a stop token may end a turn
+            k = 1
         # ---- alloc k tokens of KV per request (preempt on exhaustion) ----
         row = 0
         while row < self.Bmax:
@@ -747,6 +753,12 @@ class LLMEngine:
         the self-advancing cursors, so snapshot and restore them."""
         saved = (self.d_ids.clone(), self.d_pos.clone(),
                  self.d_seq_lens.clone(), self.d_step.clone())
+        if self.states is not None:
+            # carried state is NOT idempotent under a repeated step (the
+            # warmup would shift every live slot once more): warm up and
+            # capture with all rows inactive, which writes nothing
+            self.d_pos.fill_(-1)
+            self.d_seq_lens.zero_()
         self._capture(bucket)
         self.d_ids.copy_(saved[0])
         self.d_pos.copy_(saved[1])

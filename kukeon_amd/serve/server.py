@@ -416,7 +416,15 @@ class ModelhubClient:
 
 def main(argv: Optional[List[str]] = None) -> None:
     ap = argparse.ArgumentParser("kukeon-modelhub")
-    ap.add_argument("--model", default="llama-3-8b")
+    ap.add_argument("--model", default="llama-3-8b",
+                    help="preset name (random-init weights)")
+    ap.add_argument("--model-dir", default=None,
+                    help="checkpoint folder (config.json + "
+                         "model.safetensors); the model class follows "
+                         "config.json's architecture")
+    ap.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16",
+                    help="activation format for families that have an "
+                         "exact fp32 mode")
     ap.add_argument("--socket", default="/run/kukeon/modelhub.sock")
     ap.add_argument("--device", default=None)
     ap.add_argument("--max-model-len", type=int, default=4096)
@@ -428,17 +436,19 @@ def main(argv: Optional[List[str]] = None) -> None:
     klog.setup(logging.INFO)
     import torch
     device = args.device or ("cuda:0" if torch.cuda.is_available() else "cpu")
-    cfg = MODEL_PRESETS[args.model]()
+    from kukeon_amd.models import registry
+    if args.model_dir:
+        cfg, model = registry.load_checkpoint(args.model_dir, device=device,
+                                              dtype=args.dtype)
+        if hasattr(model, "set_max_position"):
+            model.set_max_position(args.max_model_len)
+    else:
+        cfg = registry.preset(args.model)
+        model = registry.build_model(cfg, device)
     ecfg = EngineConfig(
         max_model_len=args.max_model_len, max_sessions=args.max_sessions,
         num_kv_blocks=args.kv_blocks or (512 if device == "cpu" else 0),
         use_graphs=not args.no_graphs and device != "cpu" and not cfg.is_moe)
-    if cfg.is_moe:
-        from kukeon_amd.models.mixtral import MixtralModel
-        model = MixtralModel(cfg, device=device)
-    else:
-        from kukeon_amd.models.llama import LlamaModel
-        model = LlamaModel(cfg, device=device)
     hub = ModelhubServer(model, cfg, ecfg, args.socket, device=device)
     hub.start()
     import signal

@@ -1,0 +1,539 @@
+"""Scenarios for the Lipedra family, run by the CPU tests (reference ops,
+fp32) and the GPU tests (HIP kernels, fp32 and bf16). Every scenario builds
+a small configuration with random weights, runs it through the engine and
+compares with the plain model in lipedra_oracle.py."""
+import math
+
+import torch
+
+import lipedra_oracle as oracle
+from kukeon_amd.engine.config import EngineConfig, SamplingParams
+from kukeon_amd.engine.engine import LLMEngine
+from kukeon_amd.engine.kv_cache import SequenceKV
+from kukeon_amd.models.lipedra import LipedraConfig, LipedraModel
+
+YARN = {"factor": 4.0, "original": 64, "fast": 8.0, "slow": 1.0}
+
+
+def mixer(heads=2, kv_heads=1, dim=8, vdim=12, conv=3, diff=0.2, scale=None,
+          rot_dims=4, base=100.0, scaling=YARN, kv_from=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+         "conv": conv, "diff": diff,
+         "scale": scale if scale is not None else dim ** -0.5,
+         "rot": {"dims": rot_dims, "base": base}}
+    if scaling:
+        m["rot"]["scaling"] = dict(scaling)
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return m
+
+
+def layer(ff=24, limit=1.5, **kw):
+    return {"type": "attention", "mixer": mixer(**kw),
+            "mlp": None if ff is None else
+            {"kind": "dense", "ff": ff, "limit": limit}}
+
+
+def config(layers, width=32, vocab=40, scale=2.0, eps=1e-5):
+    return {"architecture": "Lipedra", "width": width, "vocab": vocab,
+            "embedding": {"scale": scale}, "norm": {"eps": eps},
+            "layers": layers}
+
+
+CONFIGS = {
+    # two owners, sharing layers in between, one layer without feed-forward
+    "mixed": lambda: config([
+        layer(heads=4, kv_heads=2, dim=8, vdim=12, conv=3),
+        layer(heads=4, kv_heads=2, dim=8, vdim=12, conv=3, kv_from=0,
+              ff=None),
+        layer(heads=3, kv_heads=3, dim=6, vdim=4, conv=2, rot_dims=6,
+              scaling=None, diff=0.45, ff=40, limit=0.7),
+        layer(heads=3, kv_heads=3, dim=6, vdim=4, conv=2, rot_dims=6,
+              scaling=None, kv_from=2, diff=0.1),
+        layer(heads=4, kv_heads=2, dim=8, vdim=12, conv=3, kv_from=0),
+    ], width=24, vocab=37, scale=3.0),
+    # no convolution (one tap), odd map size, value rows wider than a wave
+    "odd": lambda: config([
+        layer(heads=2, kv_heads=2, dim=7, vdim=70, conv=1, rot_dims=4),
+        layer(heads=6, kv_heads=2, dim=5, vdim=3, conv=5, rot_dims=2,
+              base=10.0, scale=0.9),
+    ], width=40, vocab=29, scale=1.0, eps=1e-3),
+    # one kv head under many query heads, long taps, full rotation
+    "gqa": lambda: config([
+        layer(heads=6, kv_heads=1, dim=16, vdim=16, conv=5, rot_dims=16),
+        layer(heads=6, kv_heads=1, dim=16, vdim=16, conv=5, rot_dims=16,
+              kv_from=0),
+    ], width=48, vocab=50, scale=0.5),
+}
+
+
+def weights(cfg, seed=0):
+    """Random checkpoint for a config dictionary, bf16 like a stored one."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+
+    def r(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16)
+
+    t = {"embed": r(cfg["vocab"], W), "final.norm": r(W, std=0.2),
+         "head": r(cfg["vocab"], W, std=W ** -0.5)}
+    for i, L in enumerate(cfg["layers"]):
+        p = "l%d." % i
+        m = L["mixer"]
+        t[p + "norm1"] = r(W, std=0.2)
+        segs = [("q", m["heads"] * 2 * m["dim"])]
+        if m.get("kv_from") is None:
+            segs += [("k", m["kv_heads"] * 2 * m["dim"]),
+                     ("v", m["kv_heads"] * m["vdim"])]
+        for n, c in segs:
+            t[p + "mix." + n] = r(c, W, std=1.5 * W ** -0.5)
+            t[p + "mix." + n + ".b"] = r(c, std=0.3)
+            t[p + "mix." + n + ".conv"] = r(c, m["conv"], std=0.6)
+        for n in ("lq1", "lk1", "lq2", "lk2"):
+            t[p + "mix." + n] = r(m["dim"], std=0.4)
+        t[p + "mix.g"] = r(m["heads"], W, std=W ** -0.5)
+        t[p + "mix.o"] = r(W, m["heads"] * m["vdim"],
+                           std=(m["heads"] * m["vdim"]) ** -0.5)
+        if L["mlp"]:
+            ff = L["mlp"]["ff"]
+            t[p + "mlp.gate"] = r(ff, W, std=2.0 * W ** -0.5)
+            t[p + "mlp.gate.b"] = r(ff, std=0.3)
+            t[p + "mlp.up"] = r(ff, W, std=2.0 * W ** -0.5)
+            t[p + "mlp.up.b"] = r(ff, std=0.3)
+            t[p + "mlp.down"] = r(W, ff, std=ff ** -0.5)
+            t[p + "mlp.down.b"] = r(W, std=0.2)
+    return t
+
+
+def tokens(cfg, n, seed):
+    g = torch.Generator().manual_seed(1000 + seed)
+    return torch.randint(0, cfg["vocab"], (n,), generator=g).tolist()
+
+
+def make_engine(cfg, tensors, device, dtype, blocks=64, slots=4,
+                block_size=4, max_len=256, poison=True):
+    mcfg = LipedraConfig.from_json(cfg)
+    model = LipedraModel(mcfg, device=device, dtype=dtype, tensors=tensors,
+                         max_position=max_len)
+    ecfg = EngineConfig(block_size=block_size, max_model_len=max_len,
+                        max_sessions=slots, state_slots=slots,
+                        num_kv_blocks=blocks, use_graphs=False)
+    eng = LLMEngine(model, mcfg, ecfg, device=device)
+    if poison:
+        # whatever a sequence has not written itself must never be read
+        for t in eng.kv.k + eng.kv.v:
+            t.fill_(300.0)
+        for t in eng.states.layers:
+            t.fill_(-700.0)
+    return eng
+
+
+def tol(dtype):
+    return 2e-4 if dtype == "fp32" else 0.08
+
+
+def rel_err(got, want):
+    """Error of logits rows as the ratio of centred root mean squares."""
+    got = got.detach().cpu().double()
+    want = want.detach().cpu().double()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    w = want - want.mean(-1, keepdim=True)
+    return float((d.pow(2).mean(-1).sqrt() /
+                  w.pow(2).mean(-1).sqrt().clamp_min(1e-9)).max())
+
+
+def check(got, want, dtype, what=""):
+    e = rel_err(got, want)
+    assert e <= tol(dtype), f"{what}: error {e:.3g} over {tol(dtype)}"
+
+
+def run_schedule(eng, prompts, schedule):
+    """schedule: list of steps, each a list of (request index, count).
+    Feeds the requests' tokens in that order; -> per request the logits at
+    every position [len, vocab]. A request is freed when it is through."""
+    bs = eng.ecfg.block_size
+    kvs, at = {}, {}
+    out = {i: [] for i in range(len(prompts))}
+    for step in schedule:
+        entries, want = [], []
+        for i, n in step:
+            if i not in kvs:
+                kvs[i] = SequenceKV(bs)
+                at[i] = 0
+            entries.append((kvs[i], prompts[i][at[i]: at[i] + n]))
+            want.append(list(range(n)))
+        lg = eng.forward_tokens(entries, want)
+        row = 0
+        for i, n in step:
+            out[i].append(lg[row: row + n])
+            row += n
+            at[i] += n
+            if at[i] == len(prompts[i]):
+                eng.free_sequence(kvs.pop(i))
+    return {i: torch.cat(v) for i, v in out.items() if v}
+
+
+def portions(total, sizes):
+    out, k = [], 0
+    while total > 0:
+        n = min(sizes[k % len(sizes)], total)
+        out.append(n)
+        total -= n
+        k += 1
+    return out
+
+
+# ---------------------------------------------------------------- scenarios
+def case_whole(name, device, dtype):
+    cfg = CONFIGS[name]()
+    W = weights(cfg, 1)
+    toks = tokens(cfg, 23, 1)
+    eng = make_engine(cfg, W, device, dtype)
+    got = run_schedule(eng, [toks], [[(0, len(toks))]])[0]
+    check(got, oracle.forward(cfg, W, toks), dtype, name)
+
+
+def case_layers(device, dtype):
+    """The residual stream after every layer."""
+    cfg = CONFIGS["mixed"]()
+    W = weights(cfg, 2)
+    toks = tokens(cfg, 9, 2)
+    eng = make_engine(cfg, W, device, dtype)
+    want = []
+    oracle.forward(cfg, W, toks, residuals=want)
+    kv = SequenceKV(eng.ecfg.block_size)
+    # the engine's packed forward with the per-layer taps switched on
+    got = []
+    fwd = eng.model.forward
+    eng.model.forward = lambda *a, **k: fwd(*a, taps=got, **k)
+    eng.forward_tokens([(kv, toks)])
+    eng.model.forward = fwd
+    assert len(got) == len(want)
+    for i, (g, w) in enumerate(zip(got, want)):
+        e = float((g.cpu().double() - w).abs().max() / w.abs().max())
+        assert e <= tol(dtype), f"layer {i}: {e:.3g}"
+
+
+def case_prefill_vs_decode(name, device, dtype):
+    cfg = CONFIGS[name]()
+    W = weights(cfg, 3)
+    toks = tokens(cfg, 21, 3)
+    want = oracle.forward(cfg, W, toks)
+    whole = run_schedule(make_engine(cfg, W, device, dtype), [toks],
+                         [[(0, len(toks))]])[0]
+    one = run_schedule(make_engine(cfg, W, device, dtype), [toks],
+                       [[(0, 1)] for _ in toks])[0]
+    check(whole, want, dtype, "whole")
+    check(one, want, dtype, "token by token")
+    check(one, whole, dtype, "token by token against whole")
+
+
+def case_portions(name, device, dtype, sizes):
+    cfg = CONFIGS[name]()
+    W = weights(cfg, 4)
+    toks = tokens(cfg, 37, 4)
+    sched = [[(0, n)] for n in portions(len(toks), sizes)]
+    got = run_schedule(make_engine(cfg, W, device, dtype), [toks], sched)[0]
+    check(got, oracle.forward(cfg, W, toks), dtype, f"portions {sizes}")
+
+
+def case_batch(name, device, dtype):
+    """Unequal requests in one batch, portions beside single tokens."""
+    cfg = CONFIGS[name]()
+    W = weights(cfg, 5)
+    prompts = [tokens(cfg, n, 10 + n) for n in (19, 1, 7, 30)]
+    sched = [
+        [(0, 5), (1, 1), (3, 2)],
+        [(0, 1), (2, 7), (3, 9)],
+        [(3, 1), (0, 1)],
+        [(0, 12), (3, 1)],
+        [(3, 17)],
+    ]
+    got = run_schedule(make_engine(cfg, W, device, dtype), prompts, sched)
+    for i, p in enumerate(prompts):
+        check(got[i], oracle.forward(cfg, W, p), dtype, f"request {i}")
+
+
+def case_reuse(device, dtype):
+    """A pool too small for all requests at once: pages and state slots of
+    finished requests are handed to the next ones."""
+    cfg = CONFIGS["mixed"]()
+    W = weights(cfg, 6)
+    prompts = [tokens(cfg, n, 20 + n) for n in (14, 11, 16, 3, 13)]
+    eng = make_engine(cfg, W, device, dtype, blocks=8, slots=2, block_size=4)
+    sched = [
+        [(0, 6), (1, 4)],
+        [(0, 8), (1, 1)],          # 0 ends: 4 pages and a slot come back
+        [(1, 6), (2, 9)],          # 1 ends
+        [(2, 7), (3, 2)],          # 2 ends
+        [(3, 1), (4, 12)],         # 3 ends
+        [(4, 1)],
+    ]
+    got = run_schedule(eng, prompts, sched)
+    for i, p in enumerate(prompts):
+        check(got[i], oracle.forward(cfg, W, p), dtype, f"request {i}")
+    assert eng.kv.allocator.num_free == 8 and eng.states.num_free == 2
+
+
+def case_first_tokens(device, dtype):
+    """Sequences shorter than the convolution, started in used slots, and a
+    start cut into single tokens."""
+    cfg = CONFIGS["gqa"]()          # 5 taps
+    W = weights(cfg, 7)
+    eng = make_engine(cfg, W, device, dtype, slots=1)
+    for n, sched in ((1, [1]), (2, [2]), (3, [1, 2]), (9, [1, 1, 1, 2, 4]),
+                     (6, [2, 1, 3])):
+        toks = tokens(cfg, n, 30 + n)
+        got = run_schedule(eng, [toks], [[(0, k)] for k in sched])[0]
+        check(got, oracle.forward(cfg, W, toks), dtype, f"length {n}")
+
+
+def case_long_decode(device, dtype):
+    cfg = CONFIGS["mixed"]()
+    W = weights(cfg, 8)
+    toks = tokens(cfg, 75, 8)
+    sched = [[(0, 3)]] + [[(0, 1)] for _ in range(72)]
+    got = run_schedule(make_engine(cfg, W, device, dtype, block_size=4),
+                       [toks], sched)[0]
+    check(got, oracle.forward(cfg, W, toks), dtype, "long decode")
+
+
+def case_greedy(device, dtype, graphs=False):
+    """Generation through add_request / step with the greedy sampler."""
+    cfg = CONFIGS["mixed"]()
+    W = weights(cfg, 9)
+    mcfg = LipedraConfig.from_json(cfg)
+    model = LipedraModel(mcfg, device=device, dtype=dtype, tensors=W,
+                         max_position=128)
+    ecfg = EngineConfig(block_size=4, max_model_len=128, max_sessions=4,
+                        state_slots=4, num_kv_blocks=64, use_graphs=graphs,
+                        graph_buckets=(4,), decode_microbatch=4,
+                        max_prefill_tokens=16)
+    eng = LLMEngine(model, mcfg, ecfg, device=device)
+    prompts = [tokens(cfg, n, 40 + n) for n in (5, 21, 2)]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=8)
+    rids = {}
+    for i, p in enumerate(prompts):
+        rids[eng.add_request(SequenceKV(4), p, sp)] = i
+    out = {i: [] for i in range(len(prompts))}
+    while eng.has_work():
+        for o in eng.step():
+            out[rids[o.req_id]].extend(o.new_tokens)
+    for i, p in enumerate(prompts):
+        want = oracle.greedy(cfg, W, p, 8)
+        if dtype == "fp32":
+            assert out[i] == want, f"request {i}: {out[i]} != {want}"
+        else:
+            # bf16 may flip a near-tie; the first tokens still agree
+            assert out[i][:2] == want[:2], f"request {i}"
+
+
+# ------------------------------------------------------- single mechanisms
+def _act(dtype):
+    return torch.float32 if dtype == "fp32" else torch.bfloat16
+
+
+def _close(got, want, dtype, what, scale=None):
+    got = got.detach().cpu().double()
+    want = want.detach().cpu().double()
+    ref = float(want.abs().max()) if scale is None else scale
+    e = float((got - want).abs().max()) / max(ref, 1e-9)
+    lim = 1e-5 if dtype == "fp32" else 2e-2
+    assert e <= lim, f"{what}: error {e:.3g} over {lim}"
+
+
+def case_op_norm(device, dtype):
+    from kukeon_amd import ops
+    g = torch.Generator().manual_seed(0)
+    for rows, W in ((5, 33), (1, 1), (3, 600)):
+        x = torch.randn(rows, W, generator=g) * 3
+        a = (torch.randn(rows, W + 3, generator=g)).to(_act(dtype))
+        b = torch.randn(W, generator=g)
+        w = torch.randn(W, generator=g) * 0.3
+        xd = x.clone().to(device)
+        out = torch.empty(rows, W, dtype=_act(dtype), device=device)
+        ops.residual_add_rmsnorm(xd, a.to(device)[:, :W], b.to(device),
+                                 w.to(device), 1.0, 1e-3, out)
+        s = x.double() + a[:, :W].double() + b.double()
+        _close(xd, s, "fp32", "residual sum")
+        _close(out, oracle.zero_centred_norm(s, w.double(), 1e-3), dtype,
+               "norm")
+        # no addend: the stream stays as it is
+        x2 = x.clone().to(device)
+        ops.residual_add_rmsnorm(x2, None, None, w.to(device), 1.0, 1e-3, out)
+        assert torch.equal(x2.cpu(), x)
+        _close(out, oracle.zero_centred_norm(x.double(), w.double(), 1e-3),
+               dtype, "norm alone")
+
+
+def case_op_glu(device, dtype):
+    from kukeon_amd import ops
+    g = torch.Generator().manual_seed(1)
+    rows, F = 7, 19
+    buf = (torch.randn(rows, 2 * F + 5, generator=g) * 3).to(_act(dtype))
+    bg = torch.randn(F, generator=g)
+    bu = torch.randn(F, generator=g)
+    d = buf.to(device)
+    out = torch.zeros(rows, F + 4, dtype=_act(dtype), device=device)
+    ops.clamp_glu(out[:, 4:], d[:, 2: 2 + F], d[:, F + 5: 2 * F + 5],
+                  bg.to(device), bu.to(device), 1.25)
+    want = oracle.clamped_glu(buf[:, 2: 2 + F].double() + bg.double(),
+                              buf[:, F + 5:].double() + bu.double(), 1.25)
+    _close(out[:, 4:], want, dtype, "clamped glu")
+    assert float(out[:, :4].abs().max()) == 0.0
+
+
+def case_op_angles():
+    from kukeon_amd.models.rotary import angle_table
+    for rot in ({"dims": 8, "base": 10000.0},
+                {"dims": 6, "base": 50.0, "scaling":
+                 {"factor": 4.0, "original": 64, "fast": 8.0, "slow": 1.0}},
+                {"dims": 16, "base": 5000.0, "scaling":
+                 {"factor": 16.0, "original": 512, "fast": 32.0,
+                  "slow": 0.5}},
+                {"dims": 2, "base": 3.0, "scaling":
+                 {"factor": 2.0, "original": 16, "fast": 4.0, "slow": 2.0}}):
+        cos, sin = oracle.rotary_angles(rot, 300)
+        t = angle_table(300, rot["dims"], rot["base"], rot.get("scaling"))
+        n = rot["dims"] // 2
+        assert float((t[:, :n].double() - cos).abs().max()) < 1e-6
+        assert float((t[:, n:].double() - sin).abs().max()) < 1e-6
+
+
+def case_op_conv_rope(device, dtype, taps=4, cuts=((5, 1, 2, 6), (3, 9))):
+    """Two sequences cut into portions; the portions of a step share one
+    launch. Checks q and what lands in the paged cache."""
+    from kukeon_amd import ops
+    from kukeon_amd.models.rotary import angle_table
+    g = torch.Generator().manual_seed(taps)
+    H, G, dim, vdim, rd, BS = 3, 2, 6, 5, 4, 4
+    Cq, Ck, Cv = H * 2 * dim, G * 2 * dim, G * vdim
+    C = Cq + Ck + Cv
+    qc, kc_, vc_ = 3, 3 + Cq + 2, 3 + Cq + 2 + Ck + 1
+    ld = vc_ + Cv + 2
+    lens = [sum(c) for c in cuts]
+    act = _act(dtype)
+    full = [(torch.randn(n, ld, generator=g)).to(act) for n in lens]
+    bias = torch.randn(C, generator=g)
+    cw = torch.randn(C, taps, generator=g) * 0.7
+    rot = {"dims": rd, "base": 30.0}
+    cs = angle_table(64, rd, 30.0, None).to(device)
+    nb = 16
+    k_cache = torch.full((nb, G, BS, 2 * dim), 99.0, dtype=act, device=device)
+    v_cache = torch.full((nb, G, BS, vdim), 99.0, dtype=act, device=device)
+    state = torch.full((3, taps - 1, C), -55.0, device=device)
+    perm = torch.randperm(nb, generator=g).tolist()
+    tables = [perm[:8], perm[8:]]
+    slots = [2, 0]
+    bt = torch.tensor(tables, dtype=torch.int32, device=device)
+    at = [0, 0]
+    q_got = [[], []]
+    nsteps = max(len(c) for c in cuts)
+    for st in range(nsteps):
+        seqs = [s for s in range(2) if st < len(cuts[s])]
+        rows, pos, rseq, cu = [], [], [], [0]
+        for k, s in enumerate(seqs):
+            n = cuts[s][st]
+            rows.append(full[s][at[s]: at[s] + n])
+            pos += list(range(at[s], at[s] + n))
+            rseq += [k] * n
+            cu.append(cu[-1] + n)
+        proj = torch.cat(rows).to(device)
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+        q_out = torch.empty(proj.shape[0], Cq, dtype=act, device=device)
+        args = (i32(pos), i32(rseq), i32(cu), i32([slots[s] for s in seqs]),
+                bt[seqs].contiguous())
+        ops.conv_rope_append(q_out, k_cache, v_cache, proj, bias.to(device),
+                             cw.to(device), state, cs, *args, qc, kc_, vc_,
+                             Cq, Ck, Cv, dim, rd)
+        ops.conv_state_update(state, proj, bias.to(device), args[0], args[2],
+                              args[3], qc, kc_, vc_, Cq, Ck, Cv)
+        for k, s in enumerate(seqs):
+            q_got[s].append(q_out[cu[k]: cu[k + 1]].cpu())
+            at[s] += cuts[s][st]
+    for s in range(2):
+        n = lens[s]
+        u = torch.cat([full[s][:, qc: qc + Cq], full[s][:, kc_: kc_ + Ck],
+                       full[s][:, vc_: vc_ + Cv]], 1).double() + bias.double()
+        y = oracle.causal_short_conv(u, cw.double())
+        cos, sin = oracle.rotary_angles(rot, n)
+        qw = oracle.rotate_interleaved(y[:, :Cq].reshape(n, 2 * H, dim), cos,
+                                       sin, rd).reshape(n, Cq)
+        kw = oracle.rotate_interleaved(
+            y[:, Cq: Cq + Ck].reshape(n, 2 * G, dim), cos, sin,
+            rd).reshape(n, G, 2 * dim)
+        vw = y[:, Cq + Ck:].reshape(n, G, vdim)
+        _close(torch.cat(q_got[s]), qw, dtype, f"q of sequence {s}")
+        kg = torch.stack([k_cache[tables[s][p // BS], :, p % BS]
+                          for p in range(n)])
+        vg = torch.stack([v_cache[tables[s][p // BS], :, p % BS]
+                          for p in range(n)])
+        _close(kg, kw, dtype, f"k of sequence {s}")
+        _close(vg, vw, dtype, f"v of sequence {s}")
+    # pages nobody owns stay untouched
+    used = set(tables[0][: -(-lens[0] // BS)] + tables[1][: -(-lens[1] // BS)])
+    for b in set(range(nb)) - used:
+        assert float((k_cache[b].float() - 99.0).abs().max()) == 0.0
+
+
+def case_op_attention_far(device, dtype, ctx=300, BS=16, H=4, G=2, dim=8,
+                          vdim=10):
+    """One key far back is made to dominate each score map (another key for
+    the second map). Keys sit at page borders; a loud key one place past the
+    query's position must stay unseen. Rows are checked as a prompt's rows
+    and as single decoded rows."""
+    from kukeon_amd import ops
+    g = torch.Generator().manual_seed(ctx + BS)
+    act = _act(dtype)
+    q = (torch.randn(ctx, H, 2, dim, generator=g) * 0.3)
+    k = (torch.randn(ctx, G, 2, dim, generator=g) * 0.3)
+    v = torch.randn(ctx, G, vdim, generator=g)
+    gate = torch.randn(ctx, H, generator=g)
+    marks = [3, BS - 1, BS, BS + 1, ctx // 2, ctx - 2]
+    probes = []
+    for n, j in enumerate(marks):
+        # the row that looks for key j, a row before j that cannot see it
+        r = min(ctx - 1, j + 5 + 37 * n)
+        axis = n % dim
+        k[j, :, 0, :] = 0
+        k[j, :, 0, axis] = 6.0
+        k[j, :, 1, :] = 0
+        q[r, :, 0, :] = 0
+        q[r, :, 0, axis] = 6.0
+        probes += [r, max(j - 1, 0), j]
+    rows = sorted(set(probes + [0, 1, ctx - 1]))
+    q, k, v, gate = (t.to(act) for t in (q, k, v, gate))
+    scale, lam, diff, eps = 0.8, 0.55, 0.3, 1e-5
+    want = oracle.diff_attention(q.double(), k.double(), v.double(), H, G,
+                                 scale, lam, diff, eps, gate.double())
+    nb = -(-ctx // BS) + 3
+    perm = torch.randperm(nb, generator=g).tolist()
+    k_cache = torch.zeros(nb, G, BS, 2 * dim, dtype=act)
+    v_cache = torch.zeros(nb, G, BS, vdim, dtype=act)
+    for p in range(ctx):
+        k_cache[perm[p // BS], :, p % BS] = k[p].reshape(G, 2 * dim)
+        v_cache[perm[p // BS], :, p % BS] = v[p]
+    bt = torch.tensor([perm, perm[::-1]], dtype=torch.int32, device=device)
+    kd, vd = k_cache.to(device), v_cache.to(device)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+
+    def run(rs):
+        out = torch.zeros(len(rs), H * vdim + 3, dtype=act, device=device)
+        ops.diff_attention(out, q[rs].reshape(len(rs), -1).to(device), kd, vd,
+                           gate[rs].to(device), i32(rs), i32([0] * len(rs)),
+                           bt, H, scale, lam, eps, 1.0 - diff)
+        return out[:, : H * vdim]
+
+    _close(run(rows), want[rows], dtype, "prompt rows", scale=1.0)
+    for r in rows:
+        _close(run([r]), want[[r]], dtype, f"decoded row {r}", scale=1.0)
+    # an inactive row (position -1) gives zeros and touches nothing else
+    out = run([rows[3], rows[4]])
+    outp = torch.zeros(2, H * vdim, dtype=act, device=device)
+    ops.diff_attention(outp, q[[rows[3], rows[4]]].reshape(2, -1).to(device),
+                       kd, vd, gate[[rows[3], rows[4]]].to(device),
+                       i32([-1, rows[4]]), i32([0, 0]), bt, H, scale, lam, eps,
+                       1.0 - diff)
+    assert float(outp[0].abs().max()) == 0.0
+    assert torch.equal(outp[1], out[1])
