@@ -420,6 +420,7 @@ class LLMEngine:
                                     for kv, _ in items])
             meta.state = self.states.layers if self.states else None
             meta.max_rows = max(len(t) for _, t in items)
+            meta.chunk_lens = [len(t) for _, t in items]
         return self.model.forward(i32(ids), self.kv.k, self.kv.v, meta)
 
     def forward_tokens(self, entries, want=None) -> torch.Tensor:

@@ -321,9 +321,7 @@ class LipedraLayer(nn.Module):
         cat = torch.empty(T, self.attn_cols + self.ff_cols, dtype=h.dtype,
                           device=h.device)
         gate = proj[:, c["g"]: c["g"] + m.heads]
-        ops.diff_attention(cat, q, kc, vc, gate, meta.positions, meta.row_seq,
-                           meta.block_table, m.heads, m.scale, self.lam,
-                           self.eps, 1.0 - m.diff)
+        self._attend(cat, q, kc, vc, gate, meta)
         if self.mlp is not None:
             ff = self.mlp.ff
             ops.clamp_glu(cat[:, self.attn_cols:],
@@ -331,6 +329,60 @@ class LipedraLayer(nn.Module):
                           proj[:, c["ffu"]: c["ffu"] + ff],
                           self.b_ffg, self.b_ffu, self.mlp.limit, 1.702, 1.0)
         return ops.linear(cat, self.w_out)
+
+
+    # ---- attention dispatch: three kernels, one contract ----
+    _ws: Dict[tuple, tuple] = {}
+
+    def _attend(self, cat, q, kc, vc, gate, meta) -> None:
+        m = self.m
+        tail = (m.heads, m.scale, self.lam, self.eps, 1.0 - m.diff)
+        rows = q.shape[0]
+        if (meta.mode == "decode" and
+                ops.diff_decode_supported(q, m.heads, m.kv_heads, m.dim,
+                                          m.vdim)):
+            # split the keys so that a small batch still fills the chip
+            ns = max(1, min(32, -(-1024 // max(1, rows * m.kv_heads))))
+            key = (q.device, rows, m.heads, ns, m.vdim)
+            ws = LipedraLayer._ws.get(key)
+            if ws is None:
+                ws = (torch.zeros(rows, m.heads, 2, ns, m.vdim,
+                                  dtype=torch.float32, device=q.device),
+                      torch.zeros(rows, m.heads, 2, ns, 2,
+                                  dtype=torch.float32, device=q.device))
+                LipedraLayer._ws[key] = ws
+            ops.diff_attention_decode(cat, q, kc, vc, gate, meta.positions,
+                                      meta.row_seq, meta.block_table, ws[0],
+                                      ws[1], *tail)
+            return
+        if (meta.mode == "prefill" and meta.max_rows >= 16 and
+                meta.chunk_lens is not None and
+                ops.diff_tiles_supported(q, m.dim, m.vdim)):
+            hpg = m.heads // m.kv_heads
+            hpw = 4 if hpg % 4 == 0 else 2 if hpg % 2 == 0 else 1
+            ts, tr = _tile_map(meta, 32 * (4 // hpw), q.device)
+            ops.diff_attention_tiles(cat, q, kc, vc, gate, meta.positions,
+                                     meta.cu_rows, meta.block_table, ts, tr,
+                                     m.heads, hpw, *tail[1:])
+            return
+        ops.diff_attention(cat, q, kc, vc, gate, meta.positions, meta.row_seq,
+                           meta.block_table, *tail)
+
+
+def _tile_map(meta, rows_per_wg: int, device):
+    """(sequence, first local row) of every workgroup of the tile kernel,
+    built once per step and granularity from the portions' lengths."""
+    cache = meta.tile_maps
+    if rows_per_wg not in cache:
+        seq, row0 = [], []
+        for s, n in enumerate(meta.chunk_lens):
+            for r in range(0, n, rows_per_wg):
+                seq.append(s)
+                row0.append(r)
+        cache[rows_per_wg] = (
+            torch.tensor(seq, dtype=torch.int32, device=device),
+            torch.tensor(row0, dtype=torch.int32, device=device))
+    return cache[rows_per_wg]
 
 
 class LipedraModel(nn.Module):

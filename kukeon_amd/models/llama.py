@@ -9,7 +9,7 @@ collective in the sampling path.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Optional
 
 import torch
@@ -43,6 +43,8 @@ class AttnMeta:
     state_slots: Optional[torch.Tensor] = None  # [nseq] int32
     state: Optional[list] = None              # per-layer state tensors
     max_rows: int = 0                         # longest portion in the batch
+    chunk_lens: Optional[list] = None         # host: rows per sequence
+    tile_maps: dict = field(default_factory=dict)  # per-step kernel maps
 
 
 def split_prefill_meta(meta: AttnMeta, parts: int = 2):

@@ -356,3 +356,36 @@ def diff_attention(out, q, k_cache, v_cache, gate, positions, row_seq,
                            gate if gate is not None else _e(q), positions,
                            row_seq, block_table, H, scale, lam, eps,
                            out_scale)
+
+
+def diff_tiles_supported(t: torch.Tensor, dim: int, vdim: int) -> bool:
+    """Whether the matrix-core kernel for prompt portions serves these
+    sizes (bf16 on a GPU only)."""
+    return (t.is_cuda and t.dtype == torch.bfloat16
+            and _mix(t).diff_attention_tiles_supported(dim, vdim))
+
+
+def diff_attention_tiles(out, q, k_cache, v_cache, gate, positions, cu_rows,
+                         block_table, tile_seq, tile_row0, H: int, hpw: int,
+                         scale: float, lam: float, eps: float,
+                         out_scale: float) -> None:
+    _mix(q).diff_attention_tiles(out, q, k_cache, v_cache,
+                                 gate if gate is not None else _e(q),
+                                 positions, cu_rows, block_table, tile_seq,
+                                 tile_row0, H, hpw, scale, lam, eps,
+                                 out_scale)
+
+
+def diff_decode_supported(t: torch.Tensor, H: int, G: int, dim: int,
+                          vdim: int) -> bool:
+    return (t.is_cuda and _mix(t).diff_attention_decode_supported(
+        H, G, dim, vdim, t.dtype == torch.bfloat16))
+
+
+def diff_attention_decode(out, q, k_cache, v_cache, gate, positions, row_seq,
+                          block_table, part_o, part_ml, H: int, scale: float,
+                          lam: float, eps: float, out_scale: float) -> None:
+    _mix(q).diff_attention_decode(out, q, k_cache, v_cache,
+                                  gate if gate is not None else _e(q),
+                                  positions, row_seq, block_table, part_o,
+                                  part_ml, H, scale, lam, eps, out_scale)

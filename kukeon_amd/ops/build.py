@@ -28,6 +28,8 @@ MIX_SOURCES = [
     "glu_clamp.hip",
     "short_conv.hip",
     "diff_attn.hip",
+    "diff_attn_mfma.hip",
+    "diff_attn_decode.hip",
     "bindings_mix.cpp",
 ]
 

@@ -30,6 +30,23 @@ void diff_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                     torch::Tensor positions, torch::Tensor row_seq,
                     torch::Tensor block_table, int64_t H, double scale,
                     double lambda, double eps, double out_scale);
+bool diff_attention_tiles_supported(int64_t dim, int64_t vdim);
+void diff_attention_tiles(torch::Tensor out, torch::Tensor q,
+                          torch::Tensor k_cache, torch::Tensor v_cache,
+                          torch::Tensor gate, torch::Tensor positions,
+                          torch::Tensor cu_rows, torch::Tensor block_table,
+                          torch::Tensor tile_seq, torch::Tensor tile_row0,
+                          int64_t H, int64_t hpw, double scale, double lambda,
+                          double eps, double out_scale);
+bool diff_attention_decode_supported(int64_t H, int64_t G, int64_t dim,
+                                     int64_t vdim, bool bf16);
+void diff_attention_decode(torch::Tensor out, torch::Tensor q,
+                           torch::Tensor k_cache, torch::Tensor v_cache,
+                           torch::Tensor gate, torch::Tensor positions,
+                           torch::Tensor row_seq, torch::Tensor block_table,
+                           torch::Tensor part_o, torch::Tensor part_ml,
+                           int64_t H, double scale, double lambda, double eps,
+                           double out_scale);
 }  // namespace kukeon
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -43,4 +60,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "shift a portion's tail into the convolution state slots");
   m.def("diff_attention", &kukeon::diff_attention,
         "paged differential attention with unit norm and output gate");
+  m.def("diff_attention_tiles_supported",
+        &kukeon::diff_attention_tiles_supported);
+  m.def("diff_attention_tiles", &kukeon::diff_attention_tiles,
+        "differential attention for prompt portions on the matrix cores");
+  m.def("diff_attention_decode_supported",
+        &kukeon::diff_attention_decode_supported);
+  m.def("diff_attention_decode", &kukeon::diff_attention_decode,
+        "split-KV differential attention for decoded rows");
 }

@@ -67,6 +67,20 @@ CONFIGS = {
 }
 
 
+# sizes the matrix-core prompt kernel serves; groups of 4, 2 and 1 heads
+CONFIGS["tiles"] = lambda: config([
+    layer(heads=4, kv_heads=1, dim=16, vdim=32, conv=3, rot_dims=8),
+    layer(heads=4, kv_heads=2, dim=32, vdim=32, conv=2, rot_dims=32,
+          scaling=None),
+    layer(heads=4, kv_heads=2, dim=32, vdim=32, conv=2, rot_dims=32,
+          scaling=None, kv_from=1),
+    layer(heads=3, kv_heads=3, dim=16, vdim=32, conv=4, rot_dims=4,
+          diff=0.4),
+    layer(heads=4, kv_heads=1, dim=16, vdim=32, conv=3, rot_dims=8,
+          kv_from=0, ff=None),
+], width=64, vocab=61, scale=1.5)
+
+
 def weights(cfg, seed=0):
     """Random checkpoint for a config dictionary, bf16 like a stored one."""
     g = torch.Generator().manual_seed(seed)
@@ -537,3 +551,62 @@ def case_op_attention_far(device, dtype, ctx=300, BS=16, H=4, G=2, dim=8,
                        1.0 - diff)
     assert float(outp[0].abs().max()) == 0.0
     assert torch.equal(outp[1], out[1])
+    if device == "cpu":
+        return
+    # the split-KV kernel for decoded rows, several split counts
+    if ops.diff_decode_supported(kd, H, G, dim, vdim):
+        for ns in (1, 3, 8):
+            rs = rows
+            po = torch.zeros(len(rs), H, 2, ns, vdim, device=device)
+            pm = torch.zeros(len(rs), H, 2, ns, 2, device=device)
+            o = torch.zeros(len(rs), H * vdim, dtype=act, device=device)
+            ps = [r if i != 1 else -1 for i, r in enumerate(rs)]
+            ops.diff_attention_decode(
+                o, q[rs].reshape(len(rs), -1).to(device), kd, vd,
+                gate[rs].to(device), i32(ps), i32([0] * len(rs)), bt, po, pm,
+                H, scale, lam, eps, 1.0 - diff)
+            assert float(o[1].abs().max()) == 0.0
+            keep = [i for i in range(len(rs)) if i != 1]
+            _close(o[keep], want[[rs[i] for i in keep]], dtype,
+                   f"split decode, {ns} splits", scale=1.0)
+    # the matrix-core kernel over the whole prompt and over its tail
+    if ops.diff_tiles_supported(kd, dim, vdim):
+        hpg = H // G
+        hpw = 4 if hpg % 4 == 0 else 2 if hpg % 2 == 0 else 1
+        step = 32 * (4 // hpw)
+        for start in (0, 37):
+            n = ctx - start
+            o = torch.zeros(n, H * vdim, dtype=act, device=device)
+            ops.diff_attention_tiles(
+                o, q[start:].reshape(n, -1).to(device), kd, vd,
+                gate[start:].to(device), i32(list(range(start, ctx))),
+                i32([0, n]), bt, i32([0] * len(range(0, n, step))),
+                i32(list(range(0, n, step))), H, hpw, scale, lam, eps,
+                1.0 - diff)
+            _close(o, want[start:], dtype, f"tile kernel from {start}",
+                   scale=1.0)
+
+
+def case_tiles(device, dtype):
+    """Prompts long enough for whole 32-row tiles, several tiles per
+    workgroup, tile edges inside pages and portions that start mid-tile."""
+    cfg = CONFIGS["tiles"]()
+    W = weights(cfg, 12)
+    prompts = [tokens(cfg, n, 50 + n) for n in (150, 33, 70, 17)]
+    want = [oracle.forward(cfg, W, p) for p in prompts]
+    eng = make_engine(cfg, W, device, dtype, blocks=96, block_size=4,
+                      max_len=256)
+    got = run_schedule(eng, prompts, [[(0, 150)], [(1, 33), (2, 70)]])
+    for i in (0, 1, 2):
+        check(got[i], want[i], dtype, f"whole {i}")
+    sched = [
+        [(0, 40), (3, 1)],
+        [(0, 31), (3, 16)],
+        [(0, 1)],
+        [(0, 64), (1, 33)],
+        [(0, 14), (2, 69)],
+        [(2, 1)],
+    ]
+    got = run_schedule(eng, prompts, sched)
+    for i in range(4):
+        check(got[i], want[i], dtype, f"portions {i}")

@@ -39,6 +39,10 @@ def test_unequal_batch(name):
     cases.case_batch(name, DEV, DT)
 
 
+def test_long_prompts_and_tile_edges():
+    cases.case_tiles(DEV, DT)
+
+
 def test_pages_and_slots_reused():
     cases.case_reuse(DEV, DT)
 

@@ -53,6 +53,11 @@ def test_unequal_batch(name, dtype):
 
 
 @BOTH
+def test_long_prompts_and_tile_edges(dtype):
+    cases.case_tiles(DEV, dtype)
+
+
+@BOTH
 def test_pages_and_slots_reused(dtype):
     cases.case_reuse(DEV, dtype)
 
@@ -93,3 +98,10 @@ def test_conv_rotary_append_op(taps, dtype):
 def test_attention_far_keys_and_page_borders(dtype):
     cases.case_op_attention_far(DEV, dtype, ctx=700, BS=16)
     cases.case_op_attention_far(DEV, dtype, ctx=70, BS=4)
+    # sizes of the matrix-core and split kernels; groups of 2, 1 and 4
+    cases.case_op_attention_far(DEV, dtype, ctx=330, BS=16, H=4, G=2,
+                                dim=16, vdim=32)
+    cases.case_op_attention_far(DEV, dtype, ctx=200, BS=8, H=2, G=2,
+                                dim=32, vdim=64)
+    cases.case_op_attention_far(DEV, dtype, ctx=130, BS=16, H=8, G=2,
+                                dim=64, vdim=128)
