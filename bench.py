@@ -21,6 +21,100 @@ import time
 import torch
 
 
+# layer sizes for --compare-families: (width, q heads, kv heads, ff, layers)
+COMPARE_SIZES = {
+    "2k": (2048, 16, 4, 8192, 4),
+    "4k": (4096, 32, 8, 14336, 4),
+    "8k": (8192, 64, 8, 28672, 2),
+}
+
+
+def compare_families(args) -> None:
+    """Prefill and decode tokens/s of Lipedra and Llama through the same
+    engine at equal sizes: same width, head counts, feed-forward size,
+    layer count, vocabulary and cache bytes per token (Llama head_dim 128;
+    Lipedra two score maps of 64 and value rows of 128)."""
+    from kukeon_amd.engine.config import (EngineConfig, ModelConfig,
+                                          SamplingParams)
+    from kukeon_amd.engine.engine import LLMEngine
+    from kukeon_amd.engine.kv_cache import SequenceKV
+    from kukeon_amd.models import registry
+    from kukeon_amd.models.lipedra import lipedra_bench
+
+    device = args.device or ("cuda:0" if torch.cuda.is_available() else "cpu")
+    on_gpu = device != "cpu"
+    nseq, plen, dlen = (32, 1024, 64) if on_gpu else (2, 40, 4)
+    vocab = 32000 if on_gpu else 512
+    rows = []
+    for size in args.compare_sizes.split(","):
+        W, hq, hk, ff, nl = COMPARE_SIZES[size]
+        if not on_gpu:
+            W, hq, hk, ff, nl = 256, 2, 2, 512, 2
+        for fam in ("llama", "lipedra"):
+            if fam == "llama":
+                cfg = ModelConfig(name=f"llama-{size}", hidden_size=W,
+                                  num_layers=nl, num_q_heads=hq,
+                                  num_kv_heads=hk, head_dim=128,
+                                  intermediate_size=ff, vocab_size=vocab,
+                                  max_position=4096)
+            else:
+                cfg = lipedra_bench(width=W, layers=nl, heads=hq,
+                                    kv_heads=hk, dim=64, vdim=128, ff=ff,
+                                    vocab=vocab, share_every=0,
+                                    name=f"lipedra-{size}")
+            model = registry.build_model(cfg, device)
+            ecfg = EngineConfig(max_model_len=2048, max_sessions=nseq,
+                                num_kv_blocks=nseq * 80 + 64,
+                                use_graphs=on_gpu and not args.no_graphs,
+                                graph_buckets=(nseq,),
+                                decode_microbatch=dlen,
+                                max_prefill_tokens=16384)
+            engine = LLMEngine(model, cfg, ecfg, device=device)
+            gen = torch.Generator().manual_seed(7)
+            sp = SamplingParams(temperature=0.7, top_k=50, top_p=0.9,
+                                max_new_tokens=dlen + 1)
+
+            def sync():
+                if on_gpu:
+                    torch.cuda.synchronize()
+
+            best = None
+            for rnd in range(1 + max(1, args.steps)):
+                kvs = [SequenceKV(ecfg.block_size) for _ in range(nseq)]
+                for kv in kvs:
+                    engine.add_request(kv, torch.randint(
+                        0, vocab, (plen,), generator=gen).tolist(), sp)
+                sync()
+                t0 = time.perf_counter()
+                while engine.waiting:
+                    engine.step()
+                sync()
+                t1 = time.perf_counter()
+                while engine.has_work():
+                    engine.step()
+                sync()
+                t2 = time.perf_counter()
+                for kv in kvs:
+                    engine.free_sequence(kv)
+                if rnd == 0:
+                    continue            # warmup: graph capture, BLAS plans
+                cur = (nseq * plen / (t1 - t0), nseq * dlen / (t2 - t1))
+                best = cur if best is None else (max(best[0], cur[0]),
+                                                 max(best[1], cur[1]))
+            rows.append({"size": size, "family": fam, "width": W,
+                         "layers": nl, "q_heads": hq, "kv_heads": hk,
+                         "ff": ff, "sequences": nseq, "prompt_len": plen,
+                         "decode_len": dlen,
+                         "prefill_tok_s": round(best[0], 1),
+                         "decode_tok_s": round(best[1], 1)})
+            del engine, model
+            if on_gpu:
+                torch.cuda.empty_cache()
+    print(json.dumps({"metric": "family_compare_tokens_per_sec",
+                      "dtype": "bf16", "data": "synthetic",
+                      "rows": rows}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -41,7 +135,16 @@ def main() -> None:
                          "across ranks, tokens routed over all-to-all "
                          "(RCCL over xGMI); sessions stay rank-local")
     ap.add_argument("--device", default=None)
+    ap.add_argument("--compare-families", action="store_true",
+                    help="instead of the headline workload: prefill and "
+                         "decode throughput of the Lipedra family beside "
+                         "Llama at equal layer sizes (random weights)")
+    ap.add_argument("--compare-sizes", default="2k,4k,8k",
+                    help="with --compare-families: which of 2k,4k,8k")
     args = ap.parse_args()
+    if args.compare_families:
+        compare_families(args)
+        return
 
     from kukeon_amd import parallel
     from kukeon_amd.engine.config import (EngineConfig, MODEL_PRESETS,

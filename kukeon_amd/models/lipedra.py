@@ -186,26 +186,21 @@ def tensor_shapes(cfg: LipedraConfig) -> Dict[str, tuple]:
 def random_tensors(cfg: LipedraConfig, seed: int = 0,
                    device="cpu") -> Dict[str, torch.Tensor]:
     """Random bf16 weights at a scale that keeps activations O(1)."""
-    g = torch.Generator(device="cpu").manual_seed(seed)
+    on_gpu = torch.device(device).type == "cuda"
+    g = torch.Generator(device=device if on_gpu else "cpu").manual_seed(seed)
+    gdev = device if on_gpu else "cpu"
     out = {}
-    big = cfg.width * cfg.vocab_size > (1 << 24)
     for name, shp in tensor_shapes(cfg).items():
-        if len(shp) == 2 and not name.endswith(".conv"):
+        leaf = name.rsplit(".", 1)[-1]
+        if len(shp) == 2 and leaf != "conv":
             std = shp[1] ** -0.5 if name != "embed" else 1.0
-            if big and torch.device(device).type == "cuda":
-                t = torch.empty(shp, dtype=torch.bfloat16, device=device)
-                t.normal_(0.0, std)
-                out[name] = t
-                continue
-            t = torch.randn(shp, generator=g) * std
-        elif name.endswith(".conv"):
-            t = torch.randn(shp, generator=g) * 0.5
-        elif name.endswith("norm1") or name == "final.norm":
-            t = torch.randn(shp, generator=g) * 0.1
-        elif name.rsplit(".", 1)[-1] in ("lq1", "lk1", "lq2", "lk2"):
-            t = torch.randn(shp, generator=g) * 0.3
+        elif leaf == "conv":
+            std = 0.5
+        elif leaf in ("lq1", "lk1", "lq2", "lk2"):
+            std = 0.3
         else:
-            t = torch.randn(shp, generator=g) * 0.1
+            std = 0.1
+        t = torch.randn(shp, generator=g, device=gdev) * std
         out[name] = t.to(torch.bfloat16).to(device)
     return out
 
