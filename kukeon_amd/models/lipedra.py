@@ -2,15 +2,17 @@
 differential-attention mixer and a clamped gated feed-forward, and both
 results join the fp32 residual stream in one sum.
 
-Per layer the compute path is two wide GEMMs and five kernels:
+Per layer the compute path is three GEMMs and five kernels:
 
   h      = rmsnorm(x) * (1 + w)                    (fused with the previous
                                                     layer's residual sum)
-  proj   = h @ [Wq | Wk | Wv | Wgate_out | Wff_gate | Wff_up]^T   (one GEMM)
+  proj   = h @ [Wq | Wk | Wv | Wgate_out]^T
+  pff    = h @ [Wff_gate | Wff_up]^T
   q,k,v  = rotary(conv(proj + bias))  -> q buffer / paged cache
   attn   = diff_attention(q, cache)   -> cat[:, :H*vdim]
-  ff     = clamp_glu(proj)            -> cat[:, H*vdim:]
-  x     += cat @ [Wo | Wdown]^T + b_down                          (one GEMM)
+  ff     = clamp_glu(pff + bias)      -> cat[:, H*vdim:]
+  x     += cat @ [Wo | Wdown]^T + b_down           (one GEMM for both
+                                                    sublayers' outputs)
 
 A layer whose mixer names `kv_from` projects no keys or values and reads
 the cache pages of that earlier layer. Everything the checkpoint's
@@ -237,25 +239,32 @@ class LipedraLayer(nn.Module):
         def w(name):
             return t[p + name].to(device=device)
 
-        # fused input projection, every segment starting on a multiple of 8
+        # two input projections off the one normed input: the mixer's
+        # [q | k | v | gate] and the feed-forward's [gate | up]; every
+        # segment starts on a multiple of 8 columns
+        def fuse(segs):
+            col, rows, at = {}, [], 0
+            for name, wt in segs:
+                col[name] = at
+                n = wt.shape[0]
+                rows.append(wt.to(dtype))
+                pad = _pad8(n) - n
+                if pad:
+                    rows.append(torch.zeros(pad, W, dtype=dtype,
+                                            device=device))
+                at += _pad8(n)
+            return col, nn.Parameter(torch.cat(rows, 0).contiguous(),
+                                     requires_grad=False)
+
         segs = [("q", w("mix.q"))]
         if self.owns_kv:
             segs += [("k", w("mix.k")), ("v", w("mix.v"))]
         segs.append(("g", w("mix.g")))
+        self.col, self.w_mix = fuse(segs)
+        self.w_ff = None
         if self.mlp is not None:
-            segs += [("ffg", w("mlp.gate")), ("ffu", w("mlp.up"))]
-        self.col = {}
-        rows, at = [], 0
-        for name, wt in segs:
-            self.col[name] = at
-            n = wt.shape[0]
-            rows.append(wt.to(dtype))
-            pad = _pad8(n) - n
-            if pad:
-                rows.append(torch.zeros(pad, W, dtype=dtype, device=device))
-            at += _pad8(n)
-        self.w_in = nn.Parameter(torch.cat(rows, 0).contiguous(),
-                                 requires_grad=False)
+            self.ffcol, self.w_ff = fuse([("ffg", w("mlp.gate")),
+                                          ("ffu", w("mlp.up"))])
         # fused output projection over [attention | feed-forward]
         outs = [w("mix.o").to(dtype)]
         self.attn_cols = m.heads * m.vdim
@@ -272,10 +281,10 @@ class LipedraLayer(nn.Module):
         # convolution taps and projection biases, fp32, channels [q|k|v]
         names = ["q"] + (["k", "v"] if self.owns_kv else [])
         self.conv_w = torch.cat([w(f"mix.{n}.conv").float() for n in names],
-                                0).contiguous()
+                                0).t().contiguous()          # [taps, C]
         self.conv_b = torch.cat([w(f"mix.{n}.b").float() for n in names],
                                 0).contiguous()
-        if self.conv_w.shape[1] != m.conv:
+        if self.conv_w.shape[0] != m.conv:
             raise ValueError(f"layer {idx}: convolution taps differ from "
                              "the configuration")
         self.norm_w = w("norm1").float().contiguous()
@@ -300,7 +309,7 @@ class LipedraLayer(nn.Module):
         kernel)."""
         m = self.m
         T = h.shape[0]
-        proj = ops.linear(h, self.w_in)
+        proj = ops.linear(h, self.w_mix)
         q = torch.empty(T, self.Cq, dtype=h.dtype, device=h.device)
         c = self.col
         ops.conv_rope_append(
@@ -319,9 +328,11 @@ class LipedraLayer(nn.Module):
         self._attend(cat, q, kc, vc, gate, meta)
         if self.mlp is not None:
             ff = self.mlp.ff
+            fc = self.ffcol
+            pff = ops.linear(h, self.w_ff)
             ops.clamp_glu(cat[:, self.attn_cols:],
-                          proj[:, c["ffg"]: c["ffg"] + ff],
-                          proj[:, c["ffu"]: c["ffu"] + ff],
+                          pff[:, fc["ffg"]: fc["ffg"] + ff],
+                          pff[:, fc["ffu"]: fc["ffu"] + ff],
                           self.b_ffg, self.b_ffu, self.mlp.limit, 1.702, 1.0)
         return ops.linear(cat, self.w_out)
 
@@ -337,7 +348,7 @@ class LipedraLayer(nn.Module):
                 ops.diff_decode_supported(q, m.heads, m.kv_heads, m.dim,
                                           m.vdim)):
             # split the keys so that a small batch still fills the chip
-            ns = max(1, min(32, -(-1024 // max(1, rows * m.kv_heads))))
+            ns = ops.diff_decode_splits(q, rows, m.heads, m.kv_heads, m.dim)
             key = (q.device, rows, m.heads, ns, m.vdim)
             ws = LipedraLayer._ws.get(key)
             if ws is None:

@@ -142,7 +142,12 @@ def _skinny5_wins(rows: int, N: int, K: int) -> bool:
     # llama-3-8b down (32.2us vs blas 39.6 cold) and llama-3-70b down
     # (79.3 vs 83.1 at M=16, 92.6 vs 139.3 at M=64) — measured on
     # MI355X, profiles/r02_progress.md
-    return (N, K) in ((4096, 14336), (8192, 28672))
+    if (N, K) in ((4096, 14336), (8192, 28672)):
+        return True
+    # the same regime — few output columns, a long reduction — that the
+    # split-K stream was built for: an output projection over a
+    # concatenated [attention | feed-forward] input
+    return N % 2048 == 0 and N <= 8192 and K % 128 == 0 and K >= 3 * N
 
 
 def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
@@ -380,6 +385,25 @@ def diff_decode_supported(t: torch.Tensor, H: int, G: int, dim: int,
                           vdim: int) -> bool:
     return (t.is_cuda and _mix(t).diff_attention_decode_supported(
         H, G, dim, vdim, t.dtype == torch.bfloat16))
+
+
+_DECODE_SPLITS = {}
+
+
+def diff_decode_splits(t: torch.Tensor, rows: int, H: int, G: int,
+                       dim: int) -> int:
+    """Split count that makes one launch exactly one full round of units
+    on the device (measured: a partly filled second round costs as much as
+    the first)."""
+    key = (t.device, t.dtype, H, G, dim)
+    cap = _DECODE_SPLITS.get(key)
+    if cap is None:
+        m = _mix(t)
+        cap = (m.diff_attention_decode_capacity(
+            H, G, dim, t.dtype == torch.bfloat16),
+            m.diff_attention_decode_units_per_row(H, G))
+        _DECODE_SPLITS[key] = cap
+    return max(1, min(32, cap[0] // max(1, rows * cap[1])))
 
 
 def diff_attention_decode(out, q, k_cache, v_cache, gate, positions, row_seq,

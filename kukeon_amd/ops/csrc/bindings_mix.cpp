@@ -40,6 +40,9 @@ void diff_attention_tiles(torch::Tensor out, torch::Tensor q,
                           double eps, double out_scale);
 bool diff_attention_decode_supported(int64_t H, int64_t G, int64_t dim,
                                      int64_t vdim, bool bf16);
+int64_t diff_attention_decode_capacity(int64_t H, int64_t G, int64_t dim,
+                                       bool bf16);
+int64_t diff_attention_decode_units_per_row(int64_t H, int64_t G);
 void diff_attention_decode(torch::Tensor out, torch::Tensor q,
                            torch::Tensor k_cache, torch::Tensor v_cache,
                            torch::Tensor gate, torch::Tensor positions,
@@ -66,6 +69,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "differential attention for prompt portions on the matrix cores");
   m.def("diff_attention_decode_supported",
         &kukeon::diff_attention_decode_supported);
+  m.def("diff_attention_decode_capacity",
+        &kukeon::diff_attention_decode_capacity);
+  m.def("diff_attention_decode_units_per_row",
+        &kukeon::diff_attention_decode_units_per_row);
   m.def("diff_attention_decode", &kukeon::diff_attention_decode,
         "split-KV differential attention for decoded rows");
 }

@@ -16,170 +16,283 @@ namespace kukeon {
 struct DecArgs {
   long ldq, ldo, ldg;
   int H, G, dim, vdim, BS, max_blocks, nsplit;
+  int hsplit;          // units per kv head: each takes (H/G)/hsplit heads
   float scale, lambda, eps, out_scale;
 };
 
-constexpr int DPASS = 256;   // keys per pass
 
-template <typename T> struct Vec16;
-template <> struct Vec16<float> {
-  static constexpr int N = 4;
-  DEV_INLINE static void load(const float* p, float* o) {
-    const float4 v = *reinterpret_cast<const float4*>(p);
-    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+// 8 raw elements of the storage format, kept unconverted while in flight
+template <typename T> struct Raw8;
+template <> struct Raw8<bf16_t> {
+  uint4 v;
+  DEV_INLINE void load(const bf16_t* p) {
+    v = *reinterpret_cast<const uint4*>(p);
+  }
+  DEV_INLINE float get(int i) const {
+    const unsigned int* w = reinterpret_cast<const unsigned int*>(&v);
+    return us2f((unsigned short)((w[i >> 1] >> ((i & 1) * 16)) & 0xffffu));
   }
 };
-template <> struct Vec16<bf16_t> {
-  static constexpr int N = 8;
-  DEV_INLINE static void load(const bf16_t* p, float* o) {
-    const bf16x8 v = load_bf16x8(p);
+template <> struct Raw8<float> {
+  float4 a, b;
+  DEV_INLINE void load(const float* p) {
+    a = *reinterpret_cast<const float4*>(p);
+    b = *reinterpret_cast<const float4*>(p + 4);
+  }
+  DEV_INLINE float get(int i) const {
+    const float* f = i < 4 ? reinterpret_cast<const float*>(&a)
+                           : reinterpret_cast<const float*>(&b);
+    return f[i & 3];
+  }
+};
+
+// Sum NV values (a power of two, <= 16) over the 16 lanes that share
+// `sub`'s upper bits. Lanes trade halves (xor 8, 4, 2, 1), so NV - 1
+// exchanges replace 4 * NV; afterwards d[0] of the lanes with index >= 0
+// holds the total of value `index`.
+template <int NV>
+DEV_INLINE int reduce_scatter16(float* d, int sub) {
+  int idx = 0;
+  int n = NV;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = v.f(i);
+  for (int mask = 8; mask >= 1; mask >>= 1) {
+    const bool up = (sub & mask) != 0;
+    if (n > 1) {
+      n >>= 1;
+#pragma unroll
+      for (int i = 0; i < NV / 2; ++i) {
+        if (i < n) {
+          const float send = up ? d[i] : d[i + n];
+          const float keep = up ? d[i + n] : d[i];
+          d[i] = keep + __shfl_xor(send, mask, WAVE);
+        }
+      }
+      idx = idx * 2 + (up ? 1 : 0);
+    } else {
+      d[0] += __shfl_xor(d[0], mask, WAVE);
+      if (up) idx = -1;                      // one writer per value
+    }
   }
-};
+  return idx;
+}
 
-template <typename T, int HP>   // HP: compile-time bound on H/G
+// One WAVE per (row, kv head, key split): the four waves of a workgroup
+// are independent units with private LDS and never meet at a barrier, so a
+// CU keeps as many splits in flight as its registers allow.
+// HP: compile-time bound on H/G; CH: 8-element pieces of a key row per lane
+// (16 lanes share a key, so a key row has at most 16 * CH pieces). A pass
+// covers P = 16 keys: every lane issues all its K and V loads of the pass
+// before using any, one HBM round trip per pass.
+template <typename T, int HP, int CH>
 __global__ __launch_bounds__(256) void diff_attn_decode_split_kernel(
     float* __restrict__ part_o,    // [rows, H, 2, nsplit, vdim]
     float* __restrict__ part_ml,   // [rows, H, 2, nsplit, 2]
     const T* __restrict__ q, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ row_seq, const int* __restrict__ block_table,
-    DecArgs a) {
+    DecArgs a, int units) {
   extern __shared__ float smem[];
-  constexpr int VN = Vec16<T>::N;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
+  constexpr int KB = 4, P = 4 * KB;         // keys per lane group / per pass
+  constexpr int WSZ = 2 * HP * P + P + 6 * HP;   // floats of LDS per wave
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int unit = blockIdx.x * 4 + wave;
+  if (unit >= units) return;
+  // units that differ only in their share of the group's heads are
+  // neighbours, so the second reader of a K/V row finds it in cache
+  const int gsub = unit % (a.G * a.hsplit);
+  const int split = (unit / (a.G * a.hsplit)) % a.nsplit;
+  const int r = unit / (a.nsplit * a.G * a.hsplit);
+  const int g = gsub / a.hsplit;
   const int dim = a.dim, vdim = a.vdim, kw = 2 * dim;
-  const int hpg = a.H / a.G;
+  const int hpg = (a.H / a.G) / a.hsplit;   // heads of this unit
+  const int h0 = g * (a.H / a.G) + (gsub % a.hsplit) * hpg;
   const int nhm = 2 * hpg;
-  float* qs = smem;                         // [hpg][kw]
-  float* sc = qs + hpg * kw;                // [2*HP][DPASS]; later partials
-  int* vrow = reinterpret_cast<int*>(sc + 2 * HP * DPASS);   // [DPASS]
-  float* st_m = reinterpret_cast<float*>(vrow + DPASS);      // [2*HP]
+  float* sc = smem + wave * WSZ;            // [2*HP][P]
+  int* vrow = reinterpret_cast<int*>(sc + 2 * HP * P);       // [P]
+  float* st_m = reinterpret_cast<float*>(vrow + P);          // [2*HP]
   float* st_l = st_m + 2 * HP;
   float* st_c = st_l + 2 * HP;
 
   const int p = positions[r];
   const int nkeys = p + 1;
   int per = nkeys > 0 ? (nkeys + a.nsplit - 1) / a.nsplit : 0;
-  per = (per + 63) / 64 * 64;
+  per = (per + P - 1) / P * P;
   const int kb = split * per;
   const int ke = kb + per < nkeys ? kb + per : nkeys;
   if (p < 0 || kb >= ke) {                  // nothing in this split
-    for (int i = tid; i < nhm; i += 256) {
-      const int h = g * hpg + i / 2, m = i & 1;
-      float* ml = part_ml + ((((long)r * a.H + h) * 2 + m) * a.nsplit + split) * 2;
+    if (lane < nhm) {
+      const int h = h0 + lane / 2, m = lane & 1;
+      float* ml = part_ml +
+                  ((((long)r * a.H + h) * 2 + m) * a.nsplit + split) * 2;
       ml[0] = -INFINITY; ml[1] = 0.f;
     }
     return;
   }
   const int* bt = block_table + (long)row_seq[r] * a.max_blocks;
-  for (int i = tid; i < hpg * kw; i += 256)
-    qs[i] = ldf(q + (long)r * a.ldq + (long)g * hpg * kw + i) * a.scale;
-  if (tid < nhm) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; }
-  __syncthreads();
-
-  const int nsl = 256 / vdim > 0 ? 256 / vdim : 1;     // vdim <= 256
-  const int pv_e = tid % vdim, pv_sl = tid / vdim;
-  const bool pv_on = tid < nsl * vdim;
-  float acc[2 * HP];
+  const int sub = lane & 15, grp = lane >> 4;
+  float qreg[HP][CH][8];
 #pragma unroll
-  for (int i = 0; i < 2 * HP; ++i) acc[i] = 0.f;
+  for (int hq = 0; hq < HP; ++hq)
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+      const int c = (sub + 16 * ch) * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qreg[hq][ch][i] = 0.f;
+      if (hq < hpg && c < kw) {
+        ld8(q + (long)r * a.ldq + (long)(h0 + hq) * kw + c,
+            qreg[hq][ch]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qreg[hq][ch][i] *= a.scale;
+      }
+    }
+  if (lane < nhm) { st_m[lane] = -INFINITY; st_l[lane] = 0.f; }
 
-  for (int j0 = kb; j0 < ke; j0 += DPASS) {
-    const int nk = ke - j0 < DPASS ? ke - j0 : DPASS;
-    // ---- scores: 4 lanes per key, 16-byte pieces of the key row ----
-    const int sub = tid & 3;
-    for (int ks = tid >> 2; ks < nk; ks += 64) {
-      const int j = j0 + ks;
-      const int vr = (bt[j / a.BS] * a.G + g) * a.BS + j % a.BS;
-      const T* kr = k_cache + (long)vr * kw;
+  const int nvec = vdim / 8;                // power of two, <= 16
+  const int nsl = 64 / nvec;                // key slices of the value step
+  const int pv_v = lane % nvec, pv_sl = lane / nvec;
+  float acc[2 * HP][8];
+#pragma unroll
+  for (int i = 0; i < 2 * HP; ++i)
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[i][k] = 0.f;
+
+  for (int j0 = kb; j0 < ke; j0 += P) {
+    const int nk = ke - j0 < P ? ke - j0 : P;
+    if (lane < nk) {
+      const int j = j0 + lane;
+      vrow[lane] = (bt[j / a.BS] * a.G + g) * a.BS + j % a.BS;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // ---- all loads of the pass ----
+    Raw8<T> kraw[KB][CH];
+#pragma unroll
+    for (int b = 0; b < KB; ++b) {
+      const int ks = grp + 4 * b < nk ? grp + 4 * b : nk - 1;
+      const T* kr = k_cache + (long)vrow[ks] * kw;
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) {
+        const int c = (sub + 16 * ch) * 8;
+        if (c < kw) kraw[b][ch].load(kr + c);
+      }
+    }
+    Raw8<T> vraw[KB];                       // P / nsl <= KB keys per lane
+#pragma unroll
+    for (int b = 0; b < KB; ++b) {
+      const int jj = pv_sl + b * nsl < nk ? pv_sl + b * nsl : nk - 1;
+      vraw[b].load(v_cache + (long)vrow[jj] * vdim + pv_v * 8);
+    }
+    // ---- scores ----
+#pragma unroll
+    for (int b = 0; b < KB; ++b) {
       float d[2 * HP];
 #pragma unroll
       for (int i = 0; i < 2 * HP; ++i) d[i] = 0.f;
-      for (int c = sub * VN; c < kw; c += 4 * VN) {
-        float kv[VN];
-        Vec16<T>::load(kr + c, kv);
-        const int m = c >= dim ? 1 : 0;       // a piece never straddles maps
 #pragma unroll
-        for (int hq = 0; hq < HP; ++hq) {
-          if (hq < hpg) {
-            const float* qq = qs + hq * kw + c;
+      for (int ch = 0; ch < CH; ++ch) {
+        const int c = (sub + 16 * ch) * 8;
+        if (c < kw) {
+          const bool second = c >= dim;     // a piece lies in one map
+          float kv[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) kv[i] = kraw[b][ch].get(i);
+#pragma unroll
+          for (int hq = 0; hq < HP; ++hq) {
             float x = 0.f;
 #pragma unroll
-            for (int i = 0; i < VN; ++i) x = fmaf(qq[i], kv[i], x);
-            if (m) d[2 * hq + 1] += x; else d[2 * hq] += x;
+            for (int i = 0; i < 8; ++i) x = fmaf(qreg[hq][ch][i], kv[i], x);
+            if (second) d[2 * hq + 1] += x; else d[2 * hq] += x;
           }
         }
       }
-#pragma unroll
-      for (int i = 0; i < 2 * HP; ++i) {
-        d[i] += __shfl_xor(d[i], 1, WAVE);
-        d[i] += __shfl_xor(d[i], 2, WAVE);
-      }
-      if (sub == 0) {
-        vrow[ks] = vr;
-#pragma unroll
-        for (int i = 0; i < 2 * HP; ++i)
-          if (i < nhm) sc[i * DPASS + ks] = d[i];
-      }
+      // reduce over the 16 lanes of the key, scattering the 2*HP sums:
+      // each exchange halves the values a lane still carries
+      const int idx = reduce_scatter16<2 * HP>(d, sub);
+      const int ks = grp + 4 * b;
+      if (idx >= 0 && idx < nhm && ks < nk) sc[idx * P + ks] = d[0];
     }
-    __syncthreads();
-    // ---- softmax statistics: one wave per (head, map) row ----
-    for (int hm = wave; hm < nhm; hm += 4) {
+    __builtin_amdgcn_wave_barrier();
+    // ---- softmax statistics: 8 lanes per (head, map) row ----
+    for (int hm = lane >> 3; hm < ((nhm + 7) & ~7); hm += 8) {
+      const int l8 = lane & 7;
+      const bool on = hm < nhm;
+      float s4[P / 8];
       float mx = -INFINITY;
-      for (int jj = lane; jj < nk; jj += 64) mx = fmaxf(mx, sc[hm * DPASS + jj]);
-      mx = wave_max(mx);
-      const float mo = st_m[hm];
+#pragma unroll
+      for (int t = 0; t < P / 8; ++t) {
+        const int jj = l8 + 8 * t;
+        s4[t] = (on && jj < nk) ? sc[hm * P + jj] : -INFINITY;
+        mx = fmaxf(mx, s4[t]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 1, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 2, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 4, WAVE));
+      const float mo = on ? st_m[hm] : 0.f;
       const float mn = fmaxf(mo, mx);
       float sum = 0.f;
-      for (int jj = lane; jj < nk; jj += 64) {
-        const float e = expf(sc[hm * DPASS + jj] - mn);
-        sc[hm * DPASS + jj] = e;
-        sum += e;
+#pragma unroll
+      for (int t = 0; t < P / 8; ++t) {
+        const int jj = l8 + 8 * t;
+        const float e = expf(s4[t] - mn);
+        if (on && jj < nk) { sc[hm * P + jj] = e; sum += e; }
       }
-      sum = wave_sum(sum);
-      if (lane == 0) {
+      sum += __shfl_xor(sum, 1, WAVE);
+      sum += __shfl_xor(sum, 2, WAVE);
+      sum += __shfl_xor(sum, 4, WAVE);
+      if (on && l8 == 0) {
         const float c = expf(mo - mn);
         st_c[hm] = c;
         st_l[hm] = st_l[hm] * c + sum;
         st_m[hm] = mn;
       }
     }
-    __syncthreads();
-    // ---- weighted values: thread (value column, key slice) ----
-    if (pv_on) {
-#pragma unroll
-      for (int i = 0; i < 2 * HP; ++i)
-        if (i < nhm) acc[i] *= st_c[i];
-      for (int jj = pv_sl; jj < nk; jj += nsl) {
-        const float v = ldf(v_cache + (long)vrow[jj] * vdim + pv_e);
-#pragma unroll
-        for (int i = 0; i < 2 * HP; ++i)
-          if (i < nhm) acc[i] = fmaf(sc[i * DPASS + jj], v, acc[i]);
-      }
-    }
-    __syncthreads();
-  }
-  // ---- fold key slices (sc is free now): part[hm][sl][e] ----
-  if (pv_on) {
+    __builtin_amdgcn_wave_barrier();
+    // ---- weighted values ----
 #pragma unroll
     for (int i = 0; i < 2 * HP; ++i)
-      if (i < nhm) sc[(i * nsl + pv_sl) * vdim + pv_e] = acc[i];
+      if (i < nhm) {
+        const float c = st_c[i];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[i][k] *= c;
+      }
+#pragma unroll
+    for (int b = 0; b < KB; ++b) {
+      const int jj = pv_sl + b * nsl;
+      if (jj < nk) {
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = vraw[b].get(k);
+#pragma unroll
+        for (int i = 0; i < 2 * HP; ++i)
+          if (i < nhm) {
+            const float w = sc[i * P + jj];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[i][k] = fmaf(w, v[k], acc[i][k]);
+          }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
   }
-  __syncthreads();
-  for (int idx = tid; idx < nhm * vdim; idx += 256) {
-    const int hm = idx / vdim, e = idx % vdim;
-    float x = 0.f;
-    for (int sl = 0; sl < nsl; ++sl) x += sc[(hm * nsl + sl) * vdim + e];
-    const int h = g * hpg + hm / 2, m = hm & 1;
-    part_o[((((long)r * a.H + h) * 2 + m) * a.nsplit + split) * vdim + e] = x;
+  // ---- fold the key slices by shuffles; lanes < nvec hold the sums ----
+#pragma unroll
+  for (int i = 0; i < 2 * HP; ++i)
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      for (int off = nvec; off < 64; off <<= 1)
+        acc[i][k] += __shfl_xor(acc[i][k], off, WAVE);
+  if (lane < nvec) {
+#pragma unroll
+    for (int i = 0; i < 2 * HP; ++i)
+      if (i < nhm) {
+        const int h = h0 + i / 2, m = i & 1;
+        st8(part_o + ((((long)r * a.H + h) * 2 + m) * a.nsplit + split) *
+                         vdim + lane * 8, acc[i]);
+      }
   }
-  if (tid < nhm) {
-    const int h = g * hpg + tid / 2, m = tid & 1;
-    float* ml = part_ml + ((((long)r * a.H + h) * 2 + m) * a.nsplit + split) * 2;
-    ml[0] = st_m[tid]; ml[1] = st_l[tid];
+  if (lane < nhm) {
+    const int h = h0 + lane / 2, m = lane & 1;
+    float* ml = part_ml +
+                ((((long)r * a.H + h) * 2 + m) * a.nsplit + split) * 2;
+    ml[0] = st_m[lane]; ml[1] = st_l[lane];
   }
 }
 
@@ -247,23 +360,31 @@ static void launch_decode(torch::Tensor& out, torch::Tensor& q,
                           torch::Tensor& gate, torch::Tensor& positions,
                           torch::Tensor& row_seq, torch::Tensor& block_table,
                           torch::Tensor& part_o, torch::Tensor& part_ml,
-                          const DecArgs& a, int HP, size_t shm,
-                          hipStream_t stream) {
+                          const DecArgs& a, int HP, int CH, int region,
+                          size_t shm, hipStream_t stream) {
   const long rows = q.size(0);
   const bool has_gate = gate.numel() > 0;
-  dim3 grid((unsigned)rows, (unsigned)a.G, (unsigned)a.nsplit);
+  const int units = (int)rows * a.G * a.hsplit * a.nsplit;
+  dim3 grid((unsigned)((units + 3) / 4));
   const T* qp = reinterpret_cast<const T*>(q.data_ptr());
   const T* kp = reinterpret_cast<const T*>(k_cache.data_ptr());
   const T* vp = reinterpret_cast<const T*>(v_cache.data_ptr());
-#define KK_DEC(N)                                                            \
-  diff_attn_decode_split_kernel<T, N><<<grid, 256, shm, stream>>>(           \
+#define KK_DEC(N, C)                                                         \
+  diff_attn_decode_split_kernel<T, N, C><<<grid, 256, shm, stream>>>(        \
       part_o.data_ptr<float>(), part_ml.data_ptr<float>(), qp, kp, vp,       \
       positions.data_ptr<int>(), row_seq.data_ptr<int>(),                    \
-      block_table.data_ptr<int>(), a)
-  if (HP == 1) KK_DEC(1);
-  else if (HP == 2) KK_DEC(2);
-  else if (HP == 4) KK_DEC(4);
-  else KK_DEC(8);
+      block_table.data_ptr<int>(), a, units)
+  if (CH == 1) {
+    if (HP == 1) KK_DEC(1, 1);
+    else if (HP == 2) KK_DEC(2, 1);
+    else if (HP == 4) KK_DEC(4, 1);
+    else KK_DEC(8, 1);
+  } else {
+    if (HP == 1) KK_DEC(1, 2);
+    else if (HP == 2) KK_DEC(2, 2);
+    else if (HP == 4) KK_DEC(4, 2);
+    else KK_DEC(8, 2);
+  }
 #undef KK_DEC
   diff_attn_decode_merge_kernel<T><<<dim3((unsigned)rows, (unsigned)a.H), 128,
                                      0, stream>>>(
@@ -273,11 +394,65 @@ static void launch_decode(torch::Tensor& out, torch::Tensor& q,
       positions.data_ptr<int>(), a);
 }
 
+static int pad_hp(int hpg) {
+  return hpg <= 1 ? 1 : hpg <= 2 ? 2 : hpg <= 4 ? 4 : 8;
+}
+
 bool diff_attention_decode_supported(int64_t H, int64_t G, int64_t dim,
                                      int64_t vdim, bool bf16) {
-  const int vn = bf16 ? 8 : 4;
-  return H % G == 0 && H / G <= 8 && dim % vn == 0 && vdim <= 256 &&
-         vdim >= 1;
+  (void)bf16;
+  if (G < 1 || H % G != 0 || H / G > 8) return false;
+  if (dim % 8 != 0 || 2 * dim > 256) return false;      // <= 32 pieces
+  if (vdim % 8 != 0) return false;
+  const int64_t nvec = vdim / 8;           // P / (64 / nvec) <= KB keys a lane
+  return nvec <= 16 && (nvec & (nvec - 1)) == 0;
+}
+
+template <typename T>
+static int64_t capacity_of(int HP, int CH, size_t shm) {
+  int blocks = 0;
+  hipError_t e = hipErrorUnknown;
+#define KK_OCC(N, C)                                                        \
+  e = hipOccupancyMaxActiveBlocksPerMultiprocessor(                         \
+      &blocks, diff_attn_decode_split_kernel<T, N, C>, 256, shm)
+  if (CH == 1) {
+    if (HP == 1) KK_OCC(1, 1); else if (HP == 2) KK_OCC(2, 1);
+    else if (HP == 4) KK_OCC(4, 1); else KK_OCC(8, 1);
+  } else {
+    if (HP == 1) KK_OCC(1, 2); else if (HP == 2) KK_OCC(2, 2);
+    else if (HP == 4) KK_OCC(4, 2); else KK_OCC(8, 2);
+  }
+#undef KK_OCC
+  if (e != hipSuccess || blocks < 1) blocks = 1;
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess)
+    hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  return (int64_t)blocks * 4 * cus;
+}
+
+static void decode_shape(int hpg_all, int dim, int* hsplit, int* HP, int* CH,
+                         size_t* shm) {
+  *hsplit = (hpg_all > 2 && hpg_all % 2 == 0) ? hpg_all / 2 : 1;
+  *HP = pad_hp(hpg_all / *hsplit);
+  *CH = 2 * dim / 8 <= 16 ? 1 : 2;
+  *shm = sizeof(float) * 4 * (size_t)(2 * *HP * 16 + 16 + 6 * *HP);
+}
+
+// How many (row, kv head share, split) units the device runs at once: the
+// caller picks the split count so that one launch is one full wave of
+// units (a second, partly filled round costs as much as the first).
+int64_t diff_attention_decode_capacity(int64_t H, int64_t G, int64_t dim,
+                                       bool bf16) {
+  int hsplit, HP, CH;
+  size_t shm;
+  decode_shape((int)(H / G), (int)dim, &hsplit, &HP, &CH, &shm);
+  return bf16 ? capacity_of<bf16_t>(HP, CH, shm)
+              : capacity_of<float>(HP, CH, shm);
+}
+
+int64_t diff_attention_decode_units_per_row(int64_t H, int64_t G) {
+  const int hpg_all = (int)(H / G);
+  return G * ((hpg_all > 2 && hpg_all % 2 == 0) ? hpg_all / 2 : 1);
 }
 
 // Same contract as diff_attention for rows that are single decoded tokens.
@@ -332,27 +507,22 @@ void diff_attention_decode(torch::Tensor out, torch::Tensor q,
   a.scale = (float)scale; a.lambda = (float)lambda; a.eps = (float)eps;
   a.out_scale = (float)out_scale;
   if (rows == 0) return;
-  const int hpg = a.H / a.G;
-  const int HP = hpg <= 1 ? 1 : hpg <= 2 ? 2 : hpg <= 4 ? 4 : 8;
-  const int nsl = 256 / a.vdim > 0 ? 256 / a.vdim : 1;
-  size_t scf = (size_t)2 * HP * DPASS;
-  const size_t fold = (size_t)2 * hpg * nsl * a.vdim;
-  if (fold > scf) scf = fold;
-  // layout in the kernel: qs | sc(2*HP*DPASS) | vrow | stats — the fold
-  // area must fit in sc
-  TORCH_CHECK(fold <= (size_t)2 * HP * DPASS,
-              "value width too large for the split decode kernel");
-  const size_t shm = sizeof(float) * ((size_t)hpg * 2 * a.dim +
-                                      (size_t)2 * HP * DPASS + DPASS +
-                                      6 * HP);
+  int HP, CH;
+  size_t shm;
+  decode_shape(a.H / a.G, a.dim, &a.hsplit, &HP, &CH, &shm);
+  const int region = 0;
   TORCH_CHECK(shm <= 64 * 1024);
+  TORCH_CHECK(aligned16(q.data_ptr()) && q.stride(0) % 8 == 0 &&
+              aligned16(k_cache.data_ptr()) && aligned16(v_cache.data_ptr()));
   auto stream = c10::hip::getCurrentHIPStream().stream();
   if (is_bf16(q))
     launch_decode<bf16_t>(out, q, k_cache, v_cache, gate, positions, row_seq,
-                          block_table, part_o, part_ml, a, HP, shm, stream);
+                          block_table, part_o, part_ml, a, HP, CH, region, shm,
+                          stream);
   else
     launch_decode<float>(out, q, k_cache, v_cache, gate, positions, row_seq,
-                         block_table, part_o, part_ml, a, HP, shm, stream);
+                         block_table, part_o, part_ml, a, HP, CH, region, shm,
+                          stream);
   HIP_CHECK_KERNEL();
 }
 

@@ -106,36 +106,58 @@ __global__ __launch_bounds__(256) void diff_attn_tile_kernel(
       for (int r = 0; r < 16; ++r) O[m][e][r] = 0.f;
   float mrun[2] = {-INFINITY, -INFINITY}, lrun[2] = {0.f, 0.f};
 
-  const int ntiles = pmax / 32 + 1;
-  for (int kt = 0; kt < ntiles; ++kt) {
-    const int k0 = kt * 32;
-    // ---- stage K (row-major) and V (transposed, keys permuted) ----
-    for (int c = tid; c < 32 * (KW / 8); c += 256) {
-      const int key = c / (KW / 8), part = c % (KW / 8);
-      const int kj = k0 + key;
-      uint4 v = uint4{0u, 0u, 0u, 0u};
-      if (kj <= pmax) {
-        const long rowi = ((long)bt[kj / a.BS] * a.G + g) * a.BS + kj % a.BS;
-        v = *reinterpret_cast<const uint4*>(k_cache + rowi * KW + part * 8);
+  // The next tile's K and V rows travel global -> registers while the
+  // current tile is being multiplied, registers -> LDS after it.
+  constexpr int KCH = 32 * (KW / 8);            // 16-byte pieces of a K tile
+  constexpr int NKC = (KCH + 255) / 256;
+  constexpr int VTASKS = 16 * (VDIM / 8);       // (key pair, 8 columns)
+  static_assert(VTASKS <= 256, "one V task per thread");
+  uint4 kreg[NKC], vreg0, vreg1;
+  const uint4 zero4 = uint4{0u, 0u, 0u, 0u};
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < NKC; ++i) {
+      const int c = tid + 256 * i;
+      kreg[i] = zero4;
+      if (c < KCH) {
+        const int kj = k0 + c / (KW / 8);
+        if (kj <= pmax) {
+          const long rowi = ((long)bt[kj / a.BS] * a.G + g) * a.BS +
+                            kj % a.BS;
+          kreg[i] = *reinterpret_cast<const uint4*>(
+              k_cache + rowi * KW + (c % (KW / 8)) * 8);
+        }
       }
-      *reinterpret_cast<uint4*>(&Ks[key * KLD + part * 8]) = v;
     }
-    for (int c = tid; c < 16 * (VDIM / 8); c += 256) {
-      const int kp = c % 16, eg = c / 16;
-      const int kj = k0 + 2 * kp;
-      uint4 v0 = uint4{0u, 0u, 0u, 0u}, v1 = v0;
+    vreg0 = zero4; vreg1 = zero4;
+    if (tid < VTASKS) {
+      const int kj = k0 + 2 * (tid % 16), eg = tid / 16;
       if (kj <= pmax) {
         const long rowi = ((long)bt[kj / a.BS] * a.G + g) * a.BS + kj % a.BS;
-        v0 = *reinterpret_cast<const uint4*>(v_cache + rowi * VDIM + eg * 8);
+        vreg0 = *reinterpret_cast<const uint4*>(v_cache + rowi * VDIM +
+                                                eg * 8);
       }
       if (kj + 1 <= pmax) {
         const int k1 = kj + 1;
         const long rowi = ((long)bt[k1 / a.BS] * a.G + g) * a.BS + k1 % a.BS;
-        v1 = *reinterpret_cast<const uint4*>(v_cache + rowi * VDIM + eg * 8);
+        vreg1 = *reinterpret_cast<const uint4*>(v_cache + rowi * VDIM +
+                                                eg * 8);
       }
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < NKC; ++i) {
+      const int c = tid + 256 * i;
+      if (c < KCH)
+        *reinterpret_cast<uint4*>(
+            &Ks[(c / (KW / 8)) * KLD + (c % (KW / 8)) * 8]) = kreg[i];
+    }
+    if (tid < VTASKS) {
+      const int kp = tid % 16, eg = tid / 16;
       const int pos = vt_pos(2 * kp);
-      const unsigned int* w0 = reinterpret_cast<const unsigned int*>(&v0);
-      const unsigned int* w1 = reinterpret_cast<const unsigned int*>(&v1);
+      const unsigned int* w0 = reinterpret_cast<const unsigned int*>(&vreg0);
+      const unsigned int* w1 = reinterpret_cast<const unsigned int*>(&vreg1);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const unsigned int lo = (w0[i >> 1] >> ((i & 1) * 16)) & 0xffffu;
@@ -144,7 +166,15 @@ __global__ __launch_bounds__(256) void diff_attn_tile_kernel(
             lo | (hi << 16);
       }
     }
+  };
+
+  const int ntiles = pmax / 32 + 1;
+  fetch(0);
+  for (int kt = 0; kt < ntiles; ++kt) {
+    const int k0 = kt * 32;
+    stash();
     __syncthreads();
+    if (kt + 1 < ntiles) fetch(k0 + 32);
 
     if (wave_on && k0 <= w_last) {
       const bool diag = k0 + 31 > w_first;

@@ -15,6 +15,29 @@ DEV_INLINE float ldf(const bf16_t* p) { return us2f(*p); }
 DEV_INLINE void stf(float* p, float v) { *p = v; }
 DEV_INLINE void stf(bf16_t* p, float v) { *p = f2us(v); }
 
+// 8 consecutive elements as fp32 (16 B of bf16, 32 B of float)
+DEV_INLINE void ld8(const float* p, float* o) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+DEV_INLINE void ld8(const bf16_t* p, float* o) {
+  const bf16x8 v = load_bf16x8(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = v.f(i);
+}
+DEV_INLINE void st8(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+  *reinterpret_cast<float4*>(p + 4) = float4{v[4], v[5], v[6], v[7]};
+}
+DEV_INLINE void st8(bf16_t* p, const float* v) {
+  *reinterpret_cast<uint4*>(p) = pack_bf16x8(v);
+}
+inline bool aligned16(const void* p) {
+  return reinterpret_cast<uintptr_t>(p) % 16 == 0;
+}
+
 // both-sum block reduction of a pair (one pass of barriers for two values)
 DEV_INLINE float2 block_sum2(float a, float b, float* red /* >= 32 floats */) {
   const int lane = threadIdx.x & (WAVE - 1);

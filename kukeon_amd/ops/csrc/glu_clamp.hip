@@ -24,6 +24,35 @@ __global__ __launch_bounds__(256) void clamp_glu_kernel(
   stf(out + r * ldo + f, g * sg * (u + up_shift));
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void clamp_glu_vec_kernel(
+    T* __restrict__ out, long ldo, const T* __restrict__ gate,
+    const T* __restrict__ up, long ldg, const float* __restrict__ bg,
+    const float* __restrict__ bu, float limit, float alpha, float up_shift,
+    int F8, long total8) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total8) return;
+  const long r = idx / F8;
+  const int f = (int)(idx - r * F8) * 8;
+  float g[8], u[8], y[8];
+  ld8(gate + r * ldg + f, g);
+  ld8(up + r * ldg + f, u);
+  if (bg) {
+    float t[8], s[8];
+    ld8(bg + f, t);
+    ld8(bu + f, s);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { g[k] += t[k]; u[k] += s[k]; }
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const float gg = fminf(g[k], limit);
+    const float uu = fminf(fmaxf(u[k], -limit), limit);
+    y[k] = gg * (1.0f / (1.0f + expf(-alpha * gg))) * (uu + up_shift);
+  }
+  st8(out + r * ldo + f, y);
+}
+
 // out [T,F] view (stride(1)==1); gate, up [T,F] views into one projection
 // buffer sharing a row stride; bg, bu [F] fp32 or empty.
 void clamp_glu(torch::Tensor out, torch::Tensor gate, torch::Tensor up,
@@ -48,6 +77,24 @@ void clamp_glu(torch::Tensor out, torch::Tensor gate, torch::Tensor up,
   const long total = rows * F;
   if (total == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  if (F % 8 == 0 && out.stride(0) % 8 == 0 && gate.stride(0) % 8 == 0 &&
+      aligned16(out.data_ptr()) && aligned16(gate.data_ptr()) &&
+      aligned16(up.data_ptr()) &&
+      (!hb || (aligned16(bg.data_ptr()) && aligned16(bu.data_ptr())))) {
+    const long total8 = total / 8;
+    KK_DISPATCH_ACT(out, {
+      clamp_glu_vec_kernel<T><<<dim3((unsigned)((total8 + 255) / 256)), 256,
+                                0, stream>>>(
+          reinterpret_cast<T*>(out.data_ptr()), out.stride(0),
+          reinterpret_cast<const T*>(gate.data_ptr()),
+          reinterpret_cast<const T*>(up.data_ptr()), gate.stride(0),
+          hb ? bg.data_ptr<float>() : nullptr,
+          hb ? bu.data_ptr<float>() : nullptr, (float)limit, (float)alpha,
+          (float)up_shift, F / 8, total8);
+    });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   KK_DISPATCH_ACT(out, {
     clamp_glu_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0,
                           stream>>>(

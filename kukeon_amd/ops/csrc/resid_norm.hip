@@ -30,6 +30,56 @@ __global__ __launch_bounds__(256) void residual_add_rmsnorm_kernel(
     stf(orow + i, xr[i] * rs * (w_offset + w[i]));
 }
 
+// Vector form: W a multiple of 8 and at most 8 * 256 * NIT; the row is held
+// in registers between the two passes and every load is 16 or 32 bytes.
+template <typename T, int NIT>
+__global__ __launch_bounds__(256) void residual_add_rmsnorm_vec_kernel(
+    float* __restrict__ x, const T* __restrict__ a, long lda,
+    const float* __restrict__ bias, const float* __restrict__ w,
+    float w_offset, float eps, T* __restrict__ out, int W) {
+  __shared__ float red[32];
+  const long row = blockIdx.x;
+  float* xr = x + row * (long)W;
+  float v[NIT][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int i = (it * 256 + threadIdx.x) * 8;
+    if (i < W) {
+      ld8(xr + i, v[it]);
+      if (a) {
+        float t[8];
+        ld8(a + row * lda + i, t);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[it][k] += t[k];
+      }
+      if (bias) {
+        float t[8];
+        ld8(bias + i, t);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[it][k] += t[k];
+      }
+      if (a || bias) st8(xr + i, v[it]);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) ss += v[it][k] * v[it][k];
+    }
+  }
+  const float2 tot = block_sum2(ss, 0.f, red);
+  const float rs = 1.0f / sqrtf(tot.x / (float)W + eps);
+  T* orow = out + row * (long)W;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int i = (it * 256 + threadIdx.x) * 8;
+    if (i < W) {
+      float t[8], o[8];
+      ld8(w + i, t);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) o[k] = v[it][k] * rs * (w_offset + t[k]);
+      st8(orow + i, o);
+    }
+  }
+}
+
 // x [T,W] fp32 (in/out); a [T,>=W] rows of stride a.stride(0) or empty;
 // bias [W] fp32 or empty; w [W] fp32; out [T,W] in the activation format.
 void residual_add_rmsnorm(torch::Tensor x, torch::Tensor a, torch::Tensor bias,
@@ -54,6 +104,36 @@ void residual_add_rmsnorm(torch::Tensor x, torch::Tensor a, torch::Tensor bias,
   }
   if (rows == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  const bool vec = W % 8 == 0 && W <= 8 * 256 * 4 && aligned16(x.data_ptr()) &&
+                   aligned16(out.data_ptr()) && aligned16(w.data_ptr()) &&
+                   (!has_a || (a.stride(0) % 8 == 0 &&
+                               aligned16(a.data_ptr()))) &&
+                   (!has_b || aligned16(bias.data_ptr()));
+  if (vec) {
+    KK_DISPATCH_ACT(out, {
+      const T* ap = has_a ? reinterpret_cast<const T*>(a.data_ptr()) : nullptr;
+      const long lda = has_a ? a.stride(0) : 0;
+      const float* bp = has_b ? bias.data_ptr<float>() : nullptr;
+      T* op = reinterpret_cast<T*>(out.data_ptr());
+      if (W <= 2048)
+        residual_add_rmsnorm_vec_kernel<T, 1><<<dim3((unsigned)rows), 256, 0,
+                                                stream>>>(
+            x.data_ptr<float>(), ap, lda, bp, w.data_ptr<float>(),
+            (float)w_offset, (float)eps, op, W);
+      else if (W <= 4096)
+        residual_add_rmsnorm_vec_kernel<T, 2><<<dim3((unsigned)rows), 256, 0,
+                                                stream>>>(
+            x.data_ptr<float>(), ap, lda, bp, w.data_ptr<float>(),
+            (float)w_offset, (float)eps, op, W);
+      else
+        residual_add_rmsnorm_vec_kernel<T, 4><<<dim3((unsigned)rows), 256, 0,
+                                                stream>>>(
+            x.data_ptr<float>(), ap, lda, bp, w.data_ptr<float>(),
+            (float)w_offset, (float)eps, op, W);
+    });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   KK_DISPATCH_ACT(out, {
     residual_add_rmsnorm_kernel<T><<<dim3((unsigned)rows), 256, 0, stream>>>(
         x.data_ptr<float>(),

@@ -6,7 +6,7 @@
 // row_seq[r] and sits at absolute position positions[r]; sequence s owns
 // rows cu_rows[s] .. cu_rows[s+1]-1 and the state slot state_slots[s].
 //   u_t[c]  = proj[t, col(c)] + bias[c]                  (fp32)
-//   y_t[c]  = sum_j cw[c, j] * u_(t - taps + 1 + j)[c]   (zeros before t=0)
+//   y_t[c]  = sum_j cw[j, c] * u_(t - taps + 1 + j)[c]   (zeros before t=0)
 // Taps that reach back before the rows of this launch are read from the
 // state slot, which keeps the last taps-1 values of u in fp32 — the same
 // numbers the in-launch path computes, so cutting a sequence into portions
@@ -49,7 +49,7 @@ DEV_INLINE float conv_channel(const T* __restrict__ proj,
       u = ldf(proj + (row0 + src) * a.ldp + col) + bias[c];
     else
       u = state_slot[(long)(back + src) * C + c];
-    acc = fmaf(cw[(long)c * a.taps + j], u, acc);
+    acc = fmaf(cw[(long)j * C + c], u, acc);
   }
   return acc;
 }
@@ -109,6 +109,88 @@ __global__ __launch_bounds__(256) void conv_rope_append_kernel(
   }
 }
 
+// Vector form: a thread owns 8 consecutive channels of one row (16-byte
+// loads and stores); a workgroup covers 32 channel groups x 8 consecutive
+// rows, so the taps that reach back into neighbouring rows hit in cache.
+// Needs every segment width, column offset, map_dim and cache row width to
+// be a multiple of 8.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_rope_append_vec_kernel(
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const T* __restrict__ proj, const float* __restrict__ bias,
+    const float* __restrict__ cw, const float* __restrict__ state,
+    const float* __restrict__ cs, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ cu_rows,
+    const int* __restrict__ state_slots, const int* __restrict__ block_table,
+    ConvArgs a, int rows) {
+  const int C = a.Cq + a.Ck + a.Cv;
+  const int cv = blockIdx.y * 32 + (threadIdx.x & 31);
+  const int r = blockIdx.x * 8 + (threadIdx.x >> 5);
+  const int c = cv * 8;
+  if (c >= C || r >= rows) return;
+  const int p = positions[r];
+  if (p < 0) return;
+  const int s = row_seq[r];
+  const long row0 = cu_rows[s];
+  const int i = r - (int)row0;
+  const int back = a.taps - 1;
+  const float* st = state + (long)state_slots[s] * back * C;
+  int seg, w;
+  long col;
+  if (c < a.Cq) { seg = 0; w = c; col = a.q_col + w; }
+  else if (c < a.Cq + a.Ck) { seg = 1; w = c - a.Cq; col = a.k_col + w; }
+  else { seg = 2; w = c - a.Cq - a.Ck; col = a.v_col + w; }
+  float b8[8], y[8];
+  ld8(bias + c, b8);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) y[k] = 0.f;
+  for (int j = 0; j < a.taps; ++j) {
+    const int src = i - back + j;
+    if (p - back + j < 0) continue;
+    float u[8], wj[8];
+    if (src >= 0) {
+      ld8(proj + (row0 + src) * a.ldp + col, u);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) u[k] += b8[k];
+    } else {
+      ld8(st + (long)(back + src) * C + c, u);
+    }
+    ld8(cw + (long)j * C + c, wj);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) y[k] = fmaf(wj[k], u[k], y[k]);
+  }
+  if (seg < 2) {
+    const int m0 = w % a.map_dim;               // multiple of 8
+    if (m0 < a.rot_dims) {
+      const int pp = p < a.cs_rows ? p : a.cs_rows - 1;
+      const float* ang = cs + (long)pp * a.rot_dims;
+#pragma unroll
+      for (int k = 0; k < 8; k += 2) {
+        if (m0 + k < a.rot_dims) {
+          const float co = ang[(m0 + k) >> 1];
+          const float si = ang[(a.rot_dims >> 1) + ((m0 + k) >> 1)];
+          const float ya = y[k], yb = y[k + 1];
+          y[k] = fmaf(-yb, si, ya * co);
+          y[k + 1] = fmaf(ya, si, yb * co);
+        }
+      }
+    }
+  }
+  if (seg == 0) {
+    st8(q_out + (long)r * a.Cq + w, y);
+    return;
+  }
+  const int blk = block_table[(long)s * a.max_blocks + p / a.BS];
+  const int off = p % a.BS;
+  if (seg == 1) {
+    const int g = w / a.kw, e = w % a.kw;
+    st8(k_cache + (((long)blk * a.G + g) * a.BS + off) * a.kw + e, y);
+  } else {
+    const int g = w / a.vw, e = w % a.vw;
+    st8(v_cache + (((long)blk * a.G + g) * a.BS + off) * a.vw + e, y);
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_update_kernel(
     float* __restrict__ state, const T* __restrict__ proj,
@@ -151,7 +233,7 @@ static ConvArgs make_args(const torch::Tensor& proj, int64_t q_col,
   return a;
 }
 
-// proj [rows, ld] (stride(1)==1); bias [C], cw [C, taps], state
+// proj [rows, ld] (stride(1)==1); bias [C], cw [taps, C], state
 // [slots, taps-1, C] fp32 with C = Cq+Ck+Cv; cs [P, rot_dims] fp32;
 // q_out [rows, Cq]; k_cache [NB, G, BS, kw], v_cache [NB, G, BS, vw] (empty
 // tensors when Ck == 0).
@@ -173,8 +255,8 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
   TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1);
   const long rows = proj.size(0);
   const long C = Cq + Ck + Cv;
-  TORCH_CHECK(cw.dim() == 2 && cw.size(0) == C && bias.numel() == C);
-  const long taps = cw.size(1);
+  TORCH_CHECK(cw.dim() == 2 && cw.size(1) == C && bias.numel() == C);
+  const long taps = cw.size(0);
   TORCH_CHECK(taps >= 1 && state.dim() == 3 && state.size(1) == taps - 1 &&
               state.size(2) == C);
   TORCH_CHECK(q_col >= 0 && q_col + Cq <= proj.size(1));
@@ -207,6 +289,32 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
   }
   if (rows == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  const bool kv = Ck > 0 || Cv > 0;
+  const bool vec =
+      Cq % 8 == 0 && Ck % 8 == 0 && Cv % 8 == 0 && q_col % 8 == 0 &&
+      (!kv || (k_col % 8 == 0 && v_col % 8 == 0 && a.kw % 8 == 0 &&
+               a.vw % 8 == 0 && aligned16(k_cache.data_ptr()) &&
+               aligned16(v_cache.data_ptr()))) &&
+      map_dim % 8 == 0 && proj.stride(0) % 8 == 0 &&
+      aligned16(proj.data_ptr()) && aligned16(q_out.data_ptr()) &&
+      aligned16(bias.data_ptr()) && aligned16(cw.data_ptr()) &&
+      aligned16(state.data_ptr());
+  if (vec) {
+    dim3 vgrid((unsigned)((rows + 7) / 8), (unsigned)((C / 8 + 31) / 32));
+    KK_DISPATCH_ACT(proj, {
+      conv_rope_append_vec_kernel<T><<<vgrid, 256, 0, stream>>>(
+          reinterpret_cast<T*>(q_out.data_ptr()),
+          Ck ? reinterpret_cast<T*>(k_cache.data_ptr()) : nullptr,
+          Cv ? reinterpret_cast<T*>(v_cache.data_ptr()) : nullptr,
+          reinterpret_cast<const T*>(proj.data_ptr()), bias.data_ptr<float>(),
+          cw.data_ptr<float>(), state.data_ptr<float>(), cs.data_ptr<float>(),
+          positions.data_ptr<int>(), row_seq.data_ptr<int>(),
+          cu_rows.data_ptr<int>(), state_slots.data_ptr<int>(),
+          block_table.data_ptr<int>(), a, (int)rows);
+    });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   dim3 grid((unsigned)rows, (unsigned)((C + 255) / 256));
   KK_DISPATCH_ACT(proj, {
     conv_rope_append_kernel<T><<<grid, 256, 0, stream>>>(

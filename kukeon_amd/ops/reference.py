@@ -291,7 +291,7 @@ def conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw, state, cs,
                      q_col: int, k_col: int, v_col: int, Cq: int, Ck: int,
                      Cv: int, map_dim: int, rot_dims: int) -> None:
     C = Cq + Ck + Cv
-    taps = cw.shape[1]
+    taps = cw.shape[0]                     # cw: [taps, C]
     back = taps - 1
     cols = _conv_cols(q_col, k_col, v_col, Cq, Ck, Cv)
     nseq = cu_rows.numel() - 1
@@ -311,7 +311,7 @@ def conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw, state, cs,
         full = torch.cat([hist, u], 0)                       # [back+n, C]
         y = torch.zeros(n, C)
         for j in range(taps):
-            y = y + cw[:, j] * full[j: j + n]
+            y = y + cw[j] * full[j: j + n]
         pos = positions[r0:r1].long()
         ang = cs[pos.clamp(max=cs.shape[0] - 1)]             # [n, rot_dims]
         half = rot_dims // 2

@@ -415,17 +415,23 @@ def case_op_angles():
         assert float((t[:, n:].double() - sin).abs().max()) < 1e-6
 
 
-def case_op_conv_rope(device, dtype, taps=4, cuts=((5, 1, 2, 6), (3, 9))):
+def case_op_conv_rope(device, dtype, taps=4, cuts=((5, 1, 2, 6), (3, 9)),
+                      aligned=False):
     """Two sequences cut into portions; the portions of a step share one
     launch. Checks q and what lands in the paged cache."""
     from kukeon_amd import ops
     from kukeon_amd.models.rotary import angle_table
     g = torch.Generator().manual_seed(taps)
     H, G, dim, vdim, rd, BS = 3, 2, 6, 5, 4, 4
+    if aligned:          # every width and offset a multiple of 8
+        H, G, dim, vdim, rd = 2, 2, 16, 8, 6
     Cq, Ck, Cv = H * 2 * dim, G * 2 * dim, G * vdim
     C = Cq + Ck + Cv
     qc, kc_, vc_ = 3, 3 + Cq + 2, 3 + Cq + 2 + Ck + 1
     ld = vc_ + Cv + 2
+    if aligned:
+        qc, kc_, vc_ = 8, 8 + Cq + 16, 8 + Cq + 16 + Ck
+        ld = vc_ + Cv + 8
     lens = [sum(c) for c in cuts]
     act = _act(dtype)
     full = [(torch.randn(n, ld, generator=g)).to(act) for n in lens]
@@ -459,7 +465,8 @@ def case_op_conv_rope(device, dtype, taps=4, cuts=((5, 1, 2, 6), (3, 9))):
         args = (i32(pos), i32(rseq), i32(cu), i32([slots[s] for s in seqs]),
                 bt[seqs].contiguous())
         ops.conv_rope_append(q_out, k_cache, v_cache, proj, bias.to(device),
-                             cw.to(device), state, cs, *args, qc, kc_, vc_,
+                             cw.t().contiguous().to(device), state, cs,
+                             *args, qc, kc_, vc_,
                              Cq, Ck, Cv, dim, rd)
         ops.conv_state_update(state, proj, bias.to(device), args[0], args[2],
                               args[3], qc, kc_, vc_, Cq, Ck, Cv)

@@ -74,6 +74,7 @@ def test_angle_tables():
 @pytest.mark.parametrize("taps", [1, 2, 4])
 def test_conv_rotary_append_op(taps):
     cases.case_op_conv_rope(DEV, DT, taps=taps)
+    cases.case_op_conv_rope(DEV, DT, taps=taps, aligned=True)
 
 
 def test_attention_far_keys_and_page_borders():

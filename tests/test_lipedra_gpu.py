@@ -92,6 +92,7 @@ def test_glu_op(dtype):
 @pytest.mark.parametrize("taps", [1, 2, 4])
 def test_conv_rotary_append_op(taps, dtype):
     cases.case_op_conv_rope(DEV, dtype, taps=taps)
+    cases.case_op_conv_rope(DEV, dtype, taps=taps, aligned=True)
 
 
 @BOTH
