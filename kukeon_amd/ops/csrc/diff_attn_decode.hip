@@ -21,31 +21,6 @@ struct DecArgs {
 };
 
 
-// 8 raw elements of the storage format, kept unconverted while in flight
-template <typename T> struct Raw8;
-template <> struct Raw8<bf16_t> {
-  uint4 v;
-  DEV_INLINE void load(const bf16_t* p) {
-    v = *reinterpret_cast<const uint4*>(p);
-  }
-  DEV_INLINE float get(int i) const {
-    const unsigned int* w = reinterpret_cast<const unsigned int*>(&v);
-    return us2f((unsigned short)((w[i >> 1] >> ((i & 1) * 16)) & 0xffffu));
-  }
-};
-template <> struct Raw8<float> {
-  float4 a, b;
-  DEV_INLINE void load(const float* p) {
-    a = *reinterpret_cast<const float4*>(p);
-    b = *reinterpret_cast<const float4*>(p + 4);
-  }
-  DEV_INLINE float get(int i) const {
-    const float* f = i < 4 ? reinterpret_cast<const float*>(&a)
-                           : reinterpret_cast<const float*>(&b);
-    return f[i & 3];
-  }
-};
-
 // Sum NV values (a power of two, <= 16) over the 16 lanes that share
 // `sub`'s upper bits. Lanes trade halves (xor 8, 4, 2, 1), so NV - 1
 // exchanges replace 4 * NV; afterwards d[0] of the lanes with index >= 0

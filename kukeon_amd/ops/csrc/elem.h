@@ -34,6 +34,31 @@ DEV_INLINE void st8(float* p, const float* v) {
 DEV_INLINE void st8(bf16_t* p, const float* v) {
   *reinterpret_cast<uint4*>(p) = pack_bf16x8(v);
 }
+// 8 raw elements of the storage format, kept unconverted while in flight
+template <typename T> struct Raw8;
+template <> struct Raw8<bf16_t> {
+  uint4 v;
+  DEV_INLINE void load(const bf16_t* p) {
+    v = *reinterpret_cast<const uint4*>(p);
+  }
+  DEV_INLINE float get(int i) const {
+    const unsigned int* w = reinterpret_cast<const unsigned int*>(&v);
+    return us2f((unsigned short)((w[i >> 1] >> ((i & 1) * 16)) & 0xffffu));
+  }
+};
+template <> struct Raw8<float> {
+  float4 a, b;
+  DEV_INLINE void load(const float* p) {
+    a = *reinterpret_cast<const float4*>(p);
+    b = *reinterpret_cast<const float4*>(p + 4);
+  }
+  DEV_INLINE float get(int i) const {
+    const float* f = i < 4 ? reinterpret_cast<const float*>(&a)
+                           : reinterpret_cast<const float*>(&b);
+    return f[i & 3];
+  }
+};
+
 inline bool aligned16(const void* p) {
   return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 }

@@ -191,6 +191,126 @@ __global__ __launch_bounds__(256) void conv_rope_append_vec_kernel(
   }
 }
 
+// Sliding form for long portions: a thread walks RB consecutive rows of its
+// 8 channels and keeps the last TAPS-1 inputs in registers, so every input
+// row is loaded once instead of TAPS times. The window is rebuilt from the
+// rows before (or the state slot) whenever a row starts another sequence.
+template <typename T, int TAPS, int RB>
+__global__ __launch_bounds__(256) void conv_rope_append_slide_kernel(
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const T* __restrict__ proj, const float* __restrict__ bias,
+    const float* __restrict__ cw, const float* __restrict__ state,
+    const float* __restrict__ cs, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ cu_rows,
+    const int* __restrict__ state_slots, const int* __restrict__ block_table,
+    ConvArgs a, int rows) {
+  constexpr int BACK = TAPS - 1;
+  const int C = a.Cq + a.Ck + a.Cv;
+  const int cv = blockIdx.y * 64 + (threadIdx.x & 63);
+  const int rb = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RB;
+  const int c = cv * 8;
+  if (c >= C || rb >= rows) return;
+  int seg, w;
+  long col;
+  if (c < a.Cq) { seg = 0; w = c; col = a.q_col + w; }
+  else if (c < a.Cq + a.Ck) { seg = 1; w = c - a.Cq; col = a.k_col + w; }
+  else { seg = 2; w = c - a.Cq - a.Ck; col = a.v_col + w; }
+  float b8[8], wt[TAPS][8], win[BACK > 0 ? BACK : 1][8];
+  ld8(bias + c, b8);
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) ld8(cw + (long)j * C + c, wt[j]);
+  const int m0 = seg < 2 ? w % a.map_dim : a.rot_dims;   // multiple of 8
+  // indices and inputs of all RB rows are requested before any is used
+  int pr[RB], sq[RB], bk[RB];
+  Raw8<T> raw[RB];
+#pragma unroll
+  for (int rr = 0; rr < RB; ++rr) {
+    const int r = rb + rr < rows ? rb + rr : rows - 1;
+    pr[rr] = rb + rr < rows ? positions[r] : -1;
+    sq[rr] = row_seq[r];
+    raw[rr].load(proj + (long)r * a.ldp + col);
+  }
+#pragma unroll
+  for (int rr = 0; rr < RB; ++rr) {
+    bk[rr] = 0;
+    if (seg > 0 && pr[rr] >= 0)
+      bk[rr] = block_table[(long)sq[rr] * a.max_blocks + pr[rr] / a.BS];
+  }
+  int prev_s = -1;
+#pragma unroll
+  for (int rr = 0; rr < RB; ++rr) {
+    const int r = rb + rr;
+    const int p = pr[rr];
+    if (p < 0) { prev_s = -1; continue; }
+    const int s = sq[rr];
+    const long row0 = cu_rows[s];
+    const int i = r - (int)row0;
+    if (s != prev_s) {                       // (re)build the window
+      const float* st = state + (long)state_slots[s] * BACK * C;
+#pragma unroll
+      for (int j = 0; j < BACK; ++j) {
+        const int src = i - BACK + j;
+        if (p - BACK + j < 0) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) win[j][k] = 0.f;
+        } else if (src >= 0) {
+          ld8(proj + (row0 + src) * a.ldp + col, win[j]);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) win[j][k] += b8[k];
+        } else {
+          ld8(st + (long)(BACK + src) * C + c, win[j]);
+        }
+      }
+      prev_s = s;
+    }
+    float u[8], y[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { u[k] = raw[rr].get(k) + b8[k]; y[k] = 0.f; }
+    // same order of accumulation as the other forms: oldest tap first
+#pragma unroll
+    for (int j = 0; j < BACK; ++j)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) y[k] = fmaf(wt[j][k], win[j][k], y[k]);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) y[k] = fmaf(wt[BACK][k], u[k], y[k]);
+#pragma unroll
+    for (int j = 0; j + 1 < BACK; ++j)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) win[j][k] = win[j + 1][k];
+    if (BACK > 0) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) win[BACK - 1][k] = u[k];
+    }
+    if (m0 < a.rot_dims) {
+      const int pp = p < a.cs_rows ? p : a.cs_rows - 1;
+      const float* ang = cs + (long)pp * a.rot_dims;
+#pragma unroll
+      for (int k = 0; k < 8; k += 2) {
+        if (m0 + k < a.rot_dims) {
+          const float co = ang[(m0 + k) >> 1];
+          const float si = ang[(a.rot_dims >> 1) + ((m0 + k) >> 1)];
+          const float ya = y[k], yb = y[k + 1];
+          y[k] = fmaf(-yb, si, ya * co);
+          y[k + 1] = fmaf(ya, si, yb * co);
+        }
+      }
+    }
+    if (seg == 0) {
+      st8(q_out + (long)r * a.Cq + w, y);
+    } else {
+      const int blk = bk[rr];
+      const int off = p % a.BS;
+      if (seg == 1) {
+        const int g = w / a.kw, e = w % a.kw;
+        st8(k_cache + (((long)blk * a.G + g) * a.BS + off) * a.kw + e, y);
+      } else {
+        const int g = w / a.vw, e = w % a.vw;
+        st8(v_cache + (((long)blk * a.G + g) * a.BS + off) * a.vw + e, y);
+      }
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_update_kernel(
     float* __restrict__ state, const T* __restrict__ proj,
@@ -299,6 +419,29 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
       aligned16(proj.data_ptr()) && aligned16(q_out.data_ptr()) &&
       aligned16(bias.data_ptr()) && aligned16(cw.data_ptr()) &&
       aligned16(state.data_ptr());
+  if (vec && rows >= 2048 && taps >= 2 && taps <= 4) {
+    constexpr int RB = 8;
+    dim3 sgrid((unsigned)((rows + 4 * RB - 1) / (4 * RB)),
+               (unsigned)((C / 8 + 63) / 64));
+#define KK_SLIDE(TP)                                                         \
+  KK_DISPATCH_ACT(proj, {                                                    \
+    conv_rope_append_slide_kernel<T, TP, RB><<<sgrid, 256, 0, stream>>>(     \
+        reinterpret_cast<T*>(q_out.data_ptr()),                              \
+        Ck ? reinterpret_cast<T*>(k_cache.data_ptr()) : nullptr,             \
+        Cv ? reinterpret_cast<T*>(v_cache.data_ptr()) : nullptr,             \
+        reinterpret_cast<const T*>(proj.data_ptr()), bias.data_ptr<float>(), \
+        cw.data_ptr<float>(), state.data_ptr<float>(), cs.data_ptr<float>(), \
+        positions.data_ptr<int>(), row_seq.data_ptr<int>(),                  \
+        cu_rows.data_ptr<int>(), state_slots.data_ptr<int>(),                \
+        block_table.data_ptr<int>(), a, (int)rows);                          \
+  })
+    if (taps == 2) KK_SLIDE(2);
+    else if (taps == 3) KK_SLIDE(3);
+    else KK_SLIDE(4);
+#undef KK_SLIDE
+    HIP_CHECK_KERNEL();
+    return;
+  }
   if (vec) {
     dim3 vgrid((unsigned)((rows + 7) / 8), (unsigned)((C / 8 + 31) / 32));
     KK_DISPATCH_ACT(proj, {

@@ -416,7 +416,7 @@ def case_op_angles():
 
 
 def case_op_conv_rope(device, dtype, taps=4, cuts=((5, 1, 2, 6), (3, 9)),
-                      aligned=False):
+                      aligned=False, pages=16):
     """Two sequences cut into portions; the portions of a step share one
     launch. Checks q and what lands in the paged cache."""
     from kukeon_amd import ops
@@ -438,13 +438,13 @@ def case_op_conv_rope(device, dtype, taps=4, cuts=((5, 1, 2, 6), (3, 9)),
     bias = torch.randn(C, generator=g)
     cw = torch.randn(C, taps, generator=g) * 0.7
     rot = {"dims": rd, "base": 30.0}
-    cs = angle_table(64, rd, 30.0, None).to(device)
-    nb = 16
+    cs = angle_table(max(64, max(lens)), rd, 30.0, None).to(device)
+    nb = pages
     k_cache = torch.full((nb, G, BS, 2 * dim), 99.0, dtype=act, device=device)
     v_cache = torch.full((nb, G, BS, vdim), 99.0, dtype=act, device=device)
     state = torch.full((3, taps - 1, C), -55.0, device=device)
     perm = torch.randperm(nb, generator=g).tolist()
-    tables = [perm[:8], perm[8:]]
+    tables = [perm[: nb // 2], perm[nb // 2:]]
     slots = [2, 0]
     bt = torch.tensor(tables, dtype=torch.int32, device=device)
     at = [0, 0]

@@ -96,6 +96,15 @@ def test_conv_rotary_append_op(taps, dtype):
 
 
 @BOTH
+@pytest.mark.parametrize("taps", [2, 3, 4])
+def test_conv_long_portions(taps, dtype):
+    """Portions long enough for the sliding-window form, a second sequence
+    starting inside a thread's run of rows, then a continuation."""
+    cases.case_op_conv_rope(DEV, dtype, taps=taps, aligned=True,
+                            cuts=((2101, 3), (150, 70)), pages=1200)
+
+
+@BOTH
 def test_attention_far_keys_and_page_borders(dtype):
     cases.case_op_attention_far(DEV, dtype, ctx=700, BS=16)
     cases.case_op_attention_far(DEV, dtype, ctx=70, BS=4)
