@@ -1,7 +1,7 @@
 """The MI355X serving engine: continuous batching over a paged KV cache.
 
 Design (MI355X-first, not a port — the reference eminwux/kukeon has no
-inference plane at all, SURVEY.md §2.9):
+inference plane at all):
 
 * one engine per GPU process; sessions own persistent KV (multi-turn agent
   context stays resident in the 288 GB HBM across turns),
@@ -270,8 +270,8 @@ class LLMEngine:
             batch, blocked = self._admit_prefill()
             # several small idle sessions may need to go before the head
             # request fits: keep evicting until admission unblocks or no
-            # victims remain (single-evict crashed on spread-out
-            # idle context even though capacity existed)
+            # victims remain (a single eviction failed on spread-out idle
+            # context even though capacity existed)
             while not batch and blocked and self._evict_idle_kv():
                 batch, blocked = self._admit_prefill()
             if batch:

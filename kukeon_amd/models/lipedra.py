@@ -337,7 +337,7 @@ class LipedraLayer(nn.Module):
         return ops.linear(cat, self.w_out)
 
 
-    # ---- attention dispatch: three kernels, one contract ----
+    # ---- attention dispatch: three kernels, one interface ----
     _ws: Dict[tuple, tuple] = {}
 
     def _attend(self, cat, q, kc, vc, gate, meta) -> None:

@@ -430,7 +430,7 @@ int64_t diff_attention_decode_units_per_row(int64_t H, int64_t G) {
   return G * ((hpg_all > 2 && hpg_all % 2 == 0) ? hpg_all / 2 : 1);
 }
 
-// Same contract as diff_attention for rows that are single decoded tokens.
+// Same arguments and result as diff_attention for rows that are single decoded tokens.
 // part_o: fp32 [rows, H, 2, nsplit, vdim]; part_ml: fp32 [rows, H, 2,
 // nsplit, 2]; nsplit <= 64.
 void diff_attention_decode(torch::Tensor out, torch::Tensor q,

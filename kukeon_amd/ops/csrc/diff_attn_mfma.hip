@@ -299,7 +299,7 @@ bool diff_attention_tiles_supported(int64_t dim, int64_t vdim) {
          (dim == 64 && vdim == 128) || (dim == 128 && vdim == 128);
 }
 
-// Same contract as diff_attention, for bf16 and the sizes listed above.
+// Same arguments and result as diff_attention, for bf16 and the sizes listed above.
 // tile_seq / tile_row0 [ntiles]: sequence and first local row of every
 // workgroup's 32 * (4 / hpw) query rows; hpw = heads per workgroup (1, 2
 // or 4, dividing H / G).

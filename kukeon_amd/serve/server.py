@@ -1,7 +1,7 @@
 """The modelhub server: the agent-backing inference service.
 
-Runs as a system-realm cell (provisioned like kukeond itself — SURVEY.md
-§2.9 integration contract): one process per GPU serving the engine over a
+Runs as a system-realm cell (provisioned like kukeond itself): one
+process per GPU serving the engine over a
 unix socket. Agent sessions hold named server-side KV contexts that stay
 resident in HBM across turns.
 
@@ -65,8 +65,7 @@ class ModelhubServer:
         self._threads = []
         self.metrics = {"tokens_generated": 0, "turns_completed": 0,
                         "engine_steps": 0, "busy_seconds": 0.0}
-        # last-N turn latencies (seconds) for the stats percentiles —
-        # the SURVEY aux-subsystem requirement (turn/latency metrics)
+        # last-N turn latencies (seconds) for the stats percentiles
         self._turn_latency = collections.deque(maxlen=512)
 
     # ---- engine loop --------------------------------------------------
