@@ -38,8 +38,16 @@ def mix_available() -> bool:
 def _mix(t: torch.Tensor):
     """Kernel group of the sequence mixers: native on a GPU tensor (an
     error if the module is not built), the fp32 references on CPU."""
+    global _C_mix, _MIX_IMPORT_ERROR
     if not t.is_cuda:
         return reference
+    if _C_mix is None:
+        # the module may have been built after this package was imported
+        try:
+            import importlib
+            _C_mix = importlib.import_module("kukeon_amd._C_mix")
+        except Exception as e:
+            _MIX_IMPORT_ERROR = e
     if _C_mix is None:
         raise RuntimeError(
             "kukeon_amd._C_mix (gfx950 HIP extension) is not built but an op "
@@ -154,6 +162,11 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """F.linear with the weight-streaming skinny-GEMM kernel on the decode
     shapes where it measured faster than hipBLASLt; hipBLASLt otherwise."""
     rows = x.shape[0]
+    if _C is None:
+        # the weight-streaming kernels are an optimisation over the vendor
+        # GEMM, not a requirement: without the core module every shape goes
+        # to the library
+        return torch.nn.functional.linear(x, w)
     if (x.is_cuda and x.dim() == 2 and rows <= 64
             and w.shape[0] % 128 == 0 and w.shape[1] % 128 == 0
             and x.dtype == torch.bfloat16
