@@ -57,11 +57,12 @@ class DiffAttnCfg:
     kv_heads: int
     dim: int                 # size of one score map of a head
     vdim: int
-    conv: int                # taps of the short convolution (1 = none)
+    conv: int                # taps of the short convolution
     diff: float
     scale: float
     rot: RotaryCfg
     kv_from: Optional[int] = None
+    has_conv: bool = True    # False: the checkpoint has no '.conv' tensors
 
 
 @dataclass
@@ -114,7 +115,8 @@ class LipedraConfig:
             mix = DiffAttnCfg(
                 heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
                 dim=int(m["dim"]), vdim=int(m["vdim"]),
-                conv=int(m.get("conv") or 1), diff=float(m["diff"]),
+                conv=int(m.get("conv") or 1),
+                has_conv=bool(m.get("conv")), diff=float(m["diff"]),
                 scale=float(m["scale"]), rot=rot,
                 kv_from=(int(m["kv_from"]) if m.get("kv_from") is not None
                          else None))
@@ -167,7 +169,8 @@ def tensor_shapes(cfg: LipedraConfig) -> Dict[str, tuple]:
         for n, c in segs:
             out[p + f"mix.{n}"] = (c, W)
             out[p + f"mix.{n}.b"] = (c,)
-            out[p + f"mix.{n}.conv"] = (c, m.conv)
+            if m.has_conv:
+                out[p + f"mix.{n}.conv"] = (c, m.conv)
         for n in ("lq1", "lk1", "lq2", "lk2"):
             out[p + "mix." + n] = (m.dim,)
         out[p + "mix.g"] = (m.heads, W)
@@ -280,8 +283,13 @@ class LipedraLayer(nn.Module):
                                   requires_grad=False)
         # convolution taps and projection biases, fp32, channels [q|k|v]
         names = ["q"] + (["k", "v"] if self.owns_kv else [])
-        self.conv_w = torch.cat([w(f"mix.{n}.conv").float() for n in names],
-                                0).t().contiguous()          # [taps, C]
+        if m.has_conv:
+            self.conv_w = torch.cat(
+                [w(f"mix.{n}.conv").float() for n in names],
+                0).t().contiguous()                          # [taps, C]
+        else:                   # no convolution: a single tap of weight 1
+            self.conv_w = torch.ones(1, self.Cq + self.Ck + self.Cv,
+                                     dtype=torch.float32, device=device)
         self.conv_b = torch.cat([w(f"mix.{n}.b").float() for n in names],
                                 0).contiguous()
         if self.conv_w.shape[0] != m.conv:

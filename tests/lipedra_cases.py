@@ -81,6 +81,25 @@ CONFIGS["tiles"] = lambda: config([
 ], width=64, vocab=61, scale=1.5)
 
 
+# a width that is no multiple of 8, no convolution key at all, 16 query
+# heads on one kv head, embedding scale left out
+def _narrow():
+    c = config([
+        layer(heads=16, kv_heads=1, dim=8, vdim=8, conv=None, rot_dims=2,
+              ff=22),
+        layer(heads=2, kv_heads=2, dim=4, vdim=6, conv=3, rot_dims=4,
+              scaling=None, ff=11, limit=0.5),
+    ], width=30, vocab=33)
+    del c["embedding"]
+    for L in c["layers"]:
+        if L["mixer"]["conv"] is None:
+            del L["mixer"]["conv"]
+    return c
+
+
+CONFIGS["narrow"] = _narrow
+
+
 def weights(cfg, seed=0):
     """Random checkpoint for a config dictionary, bf16 like a stored one."""
     g = torch.Generator().manual_seed(seed)
@@ -102,7 +121,8 @@ def weights(cfg, seed=0):
         for n, c in segs:
             t[p + "mix." + n] = r(c, W, std=1.5 * W ** -0.5)
             t[p + "mix." + n + ".b"] = r(c, std=0.3)
-            t[p + "mix." + n + ".conv"] = r(c, m["conv"], std=0.6)
+            if m.get("conv"):
+                t[p + "mix." + n + ".conv"] = r(c, m["conv"], std=0.6)
         for n in ("lq1", "lk1", "lq2", "lk2"):
             t[p + "mix." + n] = r(m["dim"], std=0.4)
         t[p + "mix.g"] = r(m["heads"], W, std=W ** -0.5)

@@ -113,6 +113,8 @@ def mixer_qkv(W, p, m, h):
 
     def proj(n):
         u = h @ W[p + "mix." + n].T + W[p + "mix." + n + ".b"]
+        if not m.get("conv"):
+            return u
         return causal_short_conv(u, W[p + "mix." + n + ".conv"])
 
     q = rotate_interleaved(proj("q").view(T, 2 * H, d), cos, sin, rd)
@@ -128,7 +130,8 @@ def forward(config, tensors, tokens, residuals=None):
     residual stream after every layer."""
     W = {k: v.to(F64) for k, v in tensors.items()}
     eps = config["norm"]["eps"]
-    x = W["embed"][torch.tensor(tokens)] * config["embedding"]["scale"]
+    x = W["embed"][torch.tensor(tokens)] * \
+        config.get("embedding", {}).get("scale", 1.0)
     held = {}
     for i, L in enumerate(config["layers"]):
         p = "l%d." % i

@@ -34,7 +34,7 @@ def test_portions_long_taps():
     cases.case_portions("gqa", DEV, DT, (2, 3))
 
 
-@pytest.mark.parametrize("name", ["mixed", "odd"])
+@pytest.mark.parametrize("name", ["mixed", "odd", "narrow"])
 def test_unequal_batch(name):
     cases.case_batch(name, DEV, DT)
 

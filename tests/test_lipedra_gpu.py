@@ -47,7 +47,7 @@ def test_portions_long_taps(dtype):
 
 
 @BOTH
-@pytest.mark.parametrize("name", ["mixed", "odd"])
+@pytest.mark.parametrize("name", ["mixed", "odd", "narrow"])
 def test_unequal_batch(name, dtype):
     cases.case_batch(name, DEV, dtype)
 
@@ -115,3 +115,9 @@ def test_attention_far_keys_and_page_borders(dtype):
                                 dim=32, vdim=64)
     cases.case_op_attention_far(DEV, dtype, ctx=130, BS=16, H=8, G=2,
                                 dim=64, vdim=128)
+    cases.case_op_attention_far(DEV, dtype, ctx=100, BS=16, H=3, G=1,
+                                dim=64, vdim=64)
+    cases.case_op_attention_far(DEV, dtype, ctx=90, BS=32, H=2, G=1,
+                                dim=128, vdim=128)
+    cases.case_op_attention_far(DEV, dtype, ctx=75, BS=16, H=16, G=2,
+                                dim=32, vdim=32)
