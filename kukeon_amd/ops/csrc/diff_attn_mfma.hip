@@ -1,10 +1,11 @@
 // Differential attention for packed prompt portions on the matrix cores
 // (bf16 operands, fp32 accumulation; gfx950 v_mfma_f32_32x32x16_bf16).
 //
-// Workgroup = 4 waves over ONE kv head: wave w serves query head
-// (w % hpw) of the group and the 32-row query tile (w / hpw), so the K and
-// V tiles staged in LDS are shared by every wave. Per 32-key tile a wave
-// computes, for both score maps,
+// Workgroup = 8 waves over ONE kv head: a pair of waves (one per score
+// map) serves query head (u % hpw) of the group and the 32-row query tile
+// (u / hpw), u = 0..3, so the K and V tiles staged in LDS are shared by
+// every wave and a wave carries one map's accumulators only. Per 32-key
+// tile a wave computes, for its map,
 //     S^T = K . Q^T           (keys x queries: a lane owns one query column,
 //                              so the softmax statistics are lane-local
 //                              plus one exchange between the half-waves)
@@ -40,29 +41,34 @@ DEV_INLINE int vt_pos(int kk) {
 }
 
 template <int DIM, int VDIM>
-__global__ __launch_bounds__(256) void diff_attn_tile_kernel(
+__global__ __launch_bounds__(512) void diff_attn_tile_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const bf16_t* __restrict__ gate, const int* __restrict__ block_table,
     const int* __restrict__ cu_rows, const int* __restrict__ positions,
     const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
     TileArgs a) {
+  constexpr int NT = 512;              // 8 waves: 4 (head, row tile) x 2 maps
   constexpr int KW = 2 * DIM;          // k row width
   constexpr int KLD = KW + 8;          // padded LDS row (bf16)
   constexpr int VLD = 40;              // 32 keys + pad
   constexpr int NC = DIM / 16;         // k-steps of the score product
   constexpr int NE = VDIM / 32;        // value row tiles
+  constexpr int XR = NE > 1 ? 2 : 1;   // rounds of the map exchange
+  constexpr int XE = NE / XR;          // value row tiles per round
   __shared__ __attribute__((aligned(16))) bf16_t Ks[32 * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vt[VDIM * VLD];
+  __shared__ float xch[4 * XE * 16 * 64];   // [unit][tile][register][lane]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
+  const int unit = wave >> 1, mp = wave & 1;   // mp: which score map
   const int col = lane & 31, hh = lane >> 5;
   const int hpg = a.H / a.G;
   const int chunks = hpg / a.hpw;
   const int g = blockIdx.y / chunks;
-  const int h = g * hpg + (blockIdx.y % chunks) * a.hpw + wave % a.hpw;
-  const int qt = wave / a.hpw;
+  const int h = g * hpg + (blockIdx.y % chunks) * a.hpw + unit % a.hpw;
+  const int qt = unit / a.hpw;
   const int QT = 4 / a.hpw;
 
   const int s = tile_seq[blockIdx.x];
@@ -80,44 +86,39 @@ __global__ __launch_bounds__(256) void diff_attn_tile_kernel(
   const int w_lastrow = (lr0 + 32 * qt + 32 < n ? lr0 + 32 * qt + 32 : n) - 1;
   const int w_last = p0 + w_lastrow;
   const int qpos = p0 + my_lr;
+  const bool row_on = wave_on && my_lr < n;
 
-  // Q fragments (B operand): query `col`, 8 contiguous dims per k-step
-  frag8_t qf[2][NC];
+  // Q fragments of this wave's map (B operand): query `col`, 8 dims a step
+  frag8_t qf[NC];
   {
-    const bool ok = wave_on && my_lr < n;
-    const bf16_t* qr = q + (long)(row_base + (ok ? my_lr : 0)) * a.ldq +
-                       (long)h * KW;
+    const bf16_t* qr = q + (long)(row_base + (row_on ? my_lr : 0)) * a.ldq +
+                       (long)h * KW + mp * DIM;
 #pragma unroll
-    for (int m = 0; m < 2; ++m)
-#pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        uint4 v = uint4{0u, 0u, 0u, 0u};
-        if (ok) v = *reinterpret_cast<const uint4*>(qr + m * DIM + 16 * c +
-                                                   8 * hh);
-        qf[m][c] = frag_of(v);
-      }
+    for (int c = 0; c < NC; ++c) {
+      uint4 v = uint4{0u, 0u, 0u, 0u};
+      if (row_on) v = *reinterpret_cast<const uint4*>(qr + 16 * c + 8 * hh);
+      qf[c] = frag_of(v);
+    }
   }
-  acc16_t O[2][NE];
+  acc16_t O[NE];
 #pragma unroll
-  for (int m = 0; m < 2; ++m)
+  for (int e = 0; e < NE; ++e)
 #pragma unroll
-    for (int e = 0; e < NE; ++e)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) O[m][e][r] = 0.f;
-  float mrun[2] = {-INFINITY, -INFINITY}, lrun[2] = {0.f, 0.f};
+    for (int r = 0; r < 16; ++r) O[e][r] = 0.f;
+  float mrun = -INFINITY, lrun = 0.f;
 
   // The next tile's K and V rows travel global -> registers while the
   // current tile is being multiplied, registers -> LDS after it.
   constexpr int KCH = 32 * (KW / 8);            // 16-byte pieces of a K tile
-  constexpr int NKC = (KCH + 255) / 256;
+  constexpr int NKC = (KCH + NT - 1) / NT;
   constexpr int VTASKS = 16 * (VDIM / 8);       // (key pair, 8 columns)
-  static_assert(VTASKS <= 256, "one V task per thread");
+  static_assert(VTASKS <= NT, "one V task per thread");
   uint4 kreg[NKC], vreg0, vreg1;
   const uint4 zero4 = uint4{0u, 0u, 0u, 0u};
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < NKC; ++i) {
-      const int c = tid + 256 * i;
+      const int c = tid + NT * i;
       kreg[i] = zero4;
       if (c < KCH) {
         const int kj = k0 + c / (KW / 8);
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(256) void diff_attn_tile_kernel(
   auto stash = [&]() {
 #pragma unroll
     for (int i = 0; i < NKC; ++i) {
-      const int c = tid + 256 * i;
+      const int c = tid + NT * i;
       if (c < KCH)
         *reinterpret_cast<uint4*>(
             &Ks[(c / (KW / 8)) * KLD + (c % (KW / 8)) * 8]) = kreg[i];
@@ -178,101 +179,111 @@ __global__ __launch_bounds__(256) void diff_attn_tile_kernel(
 
     if (wave_on && k0 <= w_last) {
       const bool diag = k0 + 31 > w_first;
-      float corr[2];
-      frag8_t ph[2][2], pl[2][2];       // [map][key half]
+      acc16_t sacc;
 #pragma unroll
-      for (int m = 0; m < 2; ++m) {
-        acc16_t sacc;
+      for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-          const frag8_t kf = frag_of(*reinterpret_cast<const uint4*>(
-              &Ks[col * KLD + m * DIM + 16 * c + 8 * hh]));
-          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[m][c], sacc,
-                                                         0, 0, 0);
-        }
-        float t[16];
-        float mx = -INFINITY;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          t[r] = sacc[r] * a.qk_log2;
-          if (diag) {
-            const int kj = k0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
-            if (kj > qpos) t[r] = -INFINITY;
-          }
-          mx = fmaxf(mx, t[r]);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-        float mn = fmaxf(mrun[m], mx);
-        if (mn == -INFINITY) mn = 0.f;           // row with no key yet
-        corr[m] = exp2f(mrun[m] - mn);
-        float sum = 0.f;
-        float p[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          p[r] = exp2f(t[r] - mn);
-          sum += p[r];
-        }
-        sum += __shfl_xor(sum, 32, WAVE);
-        lrun[m] = lrun[m] * corr[m] + sum;
-        mrun[m] = mn;
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-          unsigned int hw[4], lw[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float x0 = p[8 * t2 + 2 * i], x1 = p[8 * t2 + 2 * i + 1];
-            const unsigned short h0 = f2us(x0), h1 = f2us(x1);
-            hw[i] = (unsigned int)h0 | ((unsigned int)h1 << 16);
-            lw[i] = (unsigned int)f2us(x0 - us2f(h0)) |
-                    ((unsigned int)f2us(x1 - us2f(h1)) << 16);
-          }
-          ph[m][t2] = frag_of(uint4{hw[0], hw[1], hw[2], hw[3]});
-          pl[m][t2] = frag_of(uint4{lw[0], lw[1], lw[2], lw[3]});
-        }
+      for (int c = 0; c < NC; ++c) {
+        const frag8_t kf = frag_of(*reinterpret_cast<const uint4*>(
+            &Ks[col * KLD + mp * DIM + 16 * c + 8 * hh]));
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[c], sacc, 0, 0,
+                                                       0);
       }
+      float t[16];
+      float mx = -INFINITY;
 #pragma unroll
-      for (int m = 0; m < 2; ++m)
+      for (int r = 0; r < 16; ++r) {
+        t[r] = sacc[r] * a.qk_log2;
+        if (diag) {
+          const int kj = k0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
+          if (kj > qpos) t[r] = -INFINITY;
+        }
+        mx = fmaxf(mx, t[r]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      float mn = fmaxf(mrun, mx);
+      if (mn == -INFINITY) mn = 0.f;             // row with no key yet
+      const float corr = exp2f(mrun - mn);
+      float sum = 0.f;
+      float p[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        p[r] = exp2f(t[r] - mn);
+        sum += p[r];
+      }
+      sum += __shfl_xor(sum, 32, WAVE);
+      lrun = lrun * corr + sum;
+      mrun = mn;
+      frag8_t ph[2], pl[2];                      // [key half]
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        unsigned int hw[4], lw[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float x0 = p[8 * t2 + 2 * i], x1 = p[8 * t2 + 2 * i + 1];
+          const unsigned short h0 = f2us(x0), h1 = f2us(x1);
+          hw[i] = (unsigned int)h0 | ((unsigned int)h1 << 16);
+          lw[i] = (unsigned int)f2us(x0 - us2f(h0)) |
+                  ((unsigned int)f2us(x1 - us2f(h1)) << 16);
+        }
+        ph[t2] = frag_of(uint4{hw[0], hw[1], hw[2], hw[3]});
+        pl[t2] = frag_of(uint4{lw[0], lw[1], lw[2], lw[3]});
+      }
+      // the running maximum moves rarely after the first tiles
+      if (__any(corr != 1.0f)) {
 #pragma unroll
         for (int e = 0; e < NE; ++e)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) O[m][e][r] *= corr[m];
+          for (int r = 0; r < 16; ++r) O[e][r] *= corr;
+      }
 #pragma unroll
       for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
           const frag8_t vf = frag_of(*reinterpret_cast<const uint4*>(
               &Vt[(e * 32 + col) * VLD + 16 * t2 + 8 * hh]));
-#pragma unroll
-          for (int m = 0; m < 2; ++m) {
-            O[m][e] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                vf, ph[m][t2], O[m][e], 0, 0, 0);
-            O[m][e] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                vf, pl[m][t2], O[m][e], 0, 0, 0);
-          }
+          O[e] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, ph[t2], O[e], 0,
+                                                         0, 0);
+          O[e] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pl[t2], O[e], 0,
+                                                         0, 0);
         }
     }
     __syncthreads();
   }
 
-  if (!wave_on || my_lr >= n) {
-    // lanes without a row still join the half-wave exchange below
+  // ---- the second map's wave hands its normalised output to the first
+  // through LDS (two rounds), which forms o = a1 - lambda a2 ----
+  const float inv = lrun > 0.f ? 1.0f / lrun : 0.f;
+  float* xu = xch + unit * (XE * 16 * 64);
+#pragma unroll
+  for (int rd = 0; rd < XR; ++rd) {
+    if (mp == 1) {
+#pragma unroll
+      for (int e = 0; e < XE; ++e)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          xu[(e * 16 + r) * 64 + lane] = O[rd * XE + e][r] * inv;
+    }
+    __syncthreads();
+    if (mp == 0) {
+#pragma unroll
+      for (int e = 0; e < XE; ++e)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          O[rd * XE + e][r] = O[rd * XE + e][r] * inv -
+                              a.lambda * xu[(e * 16 + r) * 64 + lane];
+    }
+    __syncthreads();
   }
-  // ---- differential combine, unit norm, gate ----
-  const float i1 = lrun[0] > 0.f ? 1.0f / lrun[0] : 0.f;
-  const float i2 = lrun[1] > 0.f ? 1.0f / lrun[1] : 0.f;
+  if (mp == 1) return;
+  // ---- unit norm, gate, store ----
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < NE; ++e)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float o = O[0][e][r] * i1 - a.lambda * (O[1][e][r] * i2);
-      O[0][e][r] = o;
-      ss += o * o;
-    }
+    for (int r = 0; r < 16; ++r) ss += O[e][r] * O[e][r];
   ss += __shfl_xor(ss, 32, WAVE);
-  if (!wave_on || my_lr >= n) return;
+  if (!row_on) return;
   const float rs = 1.0f / sqrtf(ss / (float)VDIM + a.eps);
   float gs = 1.f;
   if (gate) {
@@ -287,8 +298,8 @@ __global__ __launch_bounds__(256) void diff_attn_tile_kernel(
     for (int r4 = 0; r4 < 4; ++r4) {
       const int e0 = e * 32 + 8 * r4 + 4 * hh;
       uint2 w;
-      w.x = cvtpk_bf16(O[0][e][4 * r4] * f, O[0][e][4 * r4 + 1] * f);
-      w.y = cvtpk_bf16(O[0][e][4 * r4 + 2] * f, O[0][e][4 * r4 + 3] * f);
+      w.x = cvtpk_bf16(O[e][4 * r4] * f, O[e][4 * r4 + 1] * f);
+      w.y = cvtpk_bf16(O[e][4 * r4 + 2] * f, O[e][4 * r4 + 3] * f);
       *reinterpret_cast<uint2*>(orow + e0) = w;
     }
 }
@@ -351,7 +362,7 @@ void diff_attention_tiles(torch::Tensor out, torch::Tensor q,
   dim3 grid((unsigned)ntiles, (unsigned)(a.G * ((a.H / a.G) / a.hpw)));
 #define KK_TILE(D, V)                                                        \
   if (dim == D && vdim == V) {                                               \
-    diff_attn_tile_kernel<D, V><<<grid, 256, 0, stream>>>(                   \
+    diff_attn_tile_kernel<D, V><<<grid, 512, 0, stream>>>(                   \
         reinterpret_cast<bf16_t*>(out.data_ptr()),                           \
         reinterpret_cast<const bf16_t*>(q.data_ptr()),                       \
         reinterpret_cast<const bf16_t*>(k_cache.data_ptr()),                 \
