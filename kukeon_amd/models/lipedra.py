@@ -320,16 +320,17 @@ class LipedraLayer(nn.Module):
         proj = ops.linear(h, self.w_mix)
         q = torch.empty(T, self.Cq, dtype=h.dtype, device=h.device)
         c = self.col
-        ops.conv_rope_append(
+        shifted = ops.conv_rope_append(
             q, kc if self.owns_kv else None, vc if self.owns_kv else None,
             proj, self.conv_b, self.conv_w, state, self.cs, meta.positions,
             meta.row_seq, meta.cu_rows, meta.state_slots, meta.block_table,
             c["q"], c.get("k", 0), c.get("v", 0), self.Cq, self.Ck, self.Cv,
-            m.dim, m.rot.dims)
-        ops.conv_state_update(state, proj, self.conv_b, meta.positions,
-                              meta.cu_rows, meta.state_slots, c["q"],
-                              c.get("k", 0), c.get("v", 0), self.Cq, self.Ck,
-                              self.Cv)
+            m.dim, m.rot.dims, one_row_per_seq=(meta.max_rows == 1))
+        if not shifted:
+            ops.conv_state_update(state, proj, self.conv_b, meta.positions,
+                                  meta.cu_rows, meta.state_slots, c["q"],
+                                  c.get("k", 0), c.get("v", 0), self.Cq,
+                                  self.Ck, self.Cv)
         cat = torch.empty(T, self.attn_cols + self.ff_cols, dtype=h.dtype,
                           device=h.device)
         gate = proj[:, c["g"]: c["g"] + m.heads]

@@ -351,13 +351,17 @@ def clamp_glu(out, gate, up, bg, bu, limit: float, alpha: float = 1.702,
 def conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw, state, cs,
                      positions, row_seq, cu_rows, state_slots, block_table,
                      q_col: int, k_col: int, v_col: int, Cq: int, Ck: int,
-                     Cv: int, map_dim: int, rot_dims: int) -> None:
+                     Cv: int, map_dim: int, rot_dims: int,
+                     one_row_per_seq: bool = False) -> bool:
+    """-> True when the state slots were shifted in the same launch (only
+    possible when every sequence brings one row); otherwise the caller
+    runs conv_state_update."""
     if k_cache is None:
         k_cache = v_cache = _e(proj)
-    _mix(proj).conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw,
-                                state, cs, positions, row_seq, cu_rows,
-                                state_slots, block_table, q_col, k_col, v_col,
-                                Cq, Ck, Cv, map_dim, rot_dims)
+    return bool(_mix(proj).conv_rope_append(
+        q_out, k_cache, v_cache, proj, bias, cw, state, cs, positions,
+        row_seq, cu_rows, state_slots, block_table, q_col, k_col, v_col,
+        Cq, Ck, Cv, map_dim, rot_dims, one_row_per_seq))
 
 
 def conv_state_update(state, proj, bias, positions, cu_rows, state_slots,

@@ -11,7 +11,7 @@ void residual_add_rmsnorm(torch::Tensor x, torch::Tensor a, torch::Tensor bias,
 void clamp_glu(torch::Tensor out, torch::Tensor gate, torch::Tensor up,
                torch::Tensor bg, torch::Tensor bu, double limit, double alpha,
                double up_shift);
-void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
+bool conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
                       torch::Tensor v_cache, torch::Tensor proj,
                       torch::Tensor bias, torch::Tensor cw,
                       torch::Tensor state, torch::Tensor cs,
@@ -19,7 +19,8 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
                       torch::Tensor cu_rows, torch::Tensor state_slots,
                       torch::Tensor block_table, int64_t q_col, int64_t k_col,
                       int64_t v_col, int64_t Cq, int64_t Ck, int64_t Cv,
-                      int64_t map_dim, int64_t rot_dims);
+                      int64_t map_dim, int64_t rot_dims,
+                      bool one_row_per_seq);
 void conv_state_update(torch::Tensor state, torch::Tensor proj,
                        torch::Tensor bias, torch::Tensor positions,
                        torch::Tensor cu_rows, torch::Tensor state_slots,

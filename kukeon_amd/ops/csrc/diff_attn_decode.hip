@@ -68,7 +68,8 @@ __global__ __launch_bounds__(256) void diff_attn_decode_split_kernel(
     DecArgs a, int units) {
   extern __shared__ float smem[];
   constexpr int KB = 4, P = 4 * KB;         // keys per lane group / per pass
-  constexpr int WSZ = 2 * HP * P + P + 6 * HP;   // floats of LDS per wave
+  constexpr int VR = 256;                   // cache rows looked up at once
+  constexpr int WSZ = 2 * HP * P + VR + 6 * HP;  // floats of LDS per wave
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int unit = blockIdx.x * 4 + wave;
   if (unit >= units) return;
@@ -83,8 +84,8 @@ __global__ __launch_bounds__(256) void diff_attn_decode_split_kernel(
   const int h0 = g * (a.H / a.G) + (gsub % a.hsplit) * hpg;
   const int nhm = 2 * hpg;
   float* sc = smem + wave * WSZ;            // [2*HP][P]
-  int* vrow = reinterpret_cast<int*>(sc + 2 * HP * P);       // [P]
-  float* st_m = reinterpret_cast<float*>(vrow + P);          // [2*HP]
+  int* vrow_all = reinterpret_cast<int*>(sc + 2 * HP * P);   // [VR]
+  float* st_m = reinterpret_cast<float*>(vrow_all + VR);     // [2*HP]
   float* st_l = st_m + 2 * HP;
   float* st_c = st_l + 2 * HP;
 
@@ -133,10 +134,19 @@ __global__ __launch_bounds__(256) void diff_attn_decode_split_kernel(
 
   for (int j0 = kb; j0 < ke; j0 += P) {
     const int nk = ke - j0 < P ? ke - j0 : P;
-    if (lane < nk) {
-      const int j = j0 + lane;
-      vrow[lane] = (bt[j / a.BS] * a.G + g) * a.BS + j % a.BS;
+    // the page lookups of the next VR keys are made together, so a pass
+    // waits on one memory round trip (its K and V rows), not two
+    if ((j0 - kb) % VR == 0) {
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int t = 0; t < VR / 64; ++t) {
+        const int j = j0 + lane + 64 * t;
+        if (j < ke)
+          vrow_all[lane + 64 * t] =
+              (bt[j / a.BS] * a.G + g) * a.BS + j % a.BS;
+      }
     }
+    const int* vrow = vrow_all + (j0 - kb) % VR;
     __builtin_amdgcn_wave_barrier();
     // ---- all loads of the pass ----
     Raw8<T> kraw[KB][CH];
@@ -410,7 +420,7 @@ static void decode_shape(int hpg_all, int dim, int* hsplit, int* HP, int* CH,
   *hsplit = (hpg_all > 2 && hpg_all % 2 == 0) ? hpg_all / 2 : 1;
   *HP = pad_hp(hpg_all / *hsplit);
   *CH = 2 * dim / 8 <= 16 ? 1 : 2;
-  *shm = sizeof(float) * 4 * (size_t)(2 * *HP * 16 + 16 + 6 * *HP);
+  *shm = sizeof(float) * 4 * (size_t)(2 * *HP * 16 + 256 + 6 * *HP);
 }
 
 // How many (row, kv head share, split) units the device runs at once: the

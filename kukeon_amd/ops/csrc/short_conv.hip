@@ -122,7 +122,7 @@ __global__ __launch_bounds__(256) void conv_rope_append_vec_kernel(
     const float* __restrict__ cs, const int* __restrict__ positions,
     const int* __restrict__ row_seq, const int* __restrict__ cu_rows,
     const int* __restrict__ state_slots, const int* __restrict__ block_table,
-    ConvArgs a, int rows) {
+    ConvArgs a, int rows, int shift_state) {
   const int C = a.Cq + a.Ck + a.Cv;
   const int cv = blockIdx.y * 32 + (threadIdx.x & 31);
   const int r = blockIdx.x * 8 + (threadIdx.x >> 5);
@@ -152,6 +152,18 @@ __global__ __launch_bounds__(256) void conv_rope_append_vec_kernel(
       ld8(proj + (row0 + src) * a.ldp + col, u);
 #pragma unroll
       for (int k = 0; k < 8; ++k) u[k] += b8[k];
+      if (shift_state && j == back) {
+        // every sequence brings one row: this thread alone owns the
+        // slot's 8 channels, so it shifts them here (all reads of the
+        // slot were made in earlier iterations of this loop)
+        float* sw = const_cast<float*>(st);
+        for (int t = 0; t + 1 < back; ++t) {
+          float m[8];
+          ld8(sw + (long)(t + 1) * C + c, m);
+          st8(sw + (long)t * C + c, m);
+        }
+        if (back > 0) st8(sw + (long)(back - 1) * C + c, u);
+      }
     } else {
       ld8(st + (long)(back + src) * C + c, u);
     }
@@ -353,11 +365,13 @@ static ConvArgs make_args(const torch::Tensor& proj, int64_t q_col,
   return a;
 }
 
+// Returns true when the kernel also shifted the state slots (one row per
+// sequence, vector form) so that no conv_state_update launch is needed.
 // proj [rows, ld] (stride(1)==1); bias [C], cw [taps, C], state
 // [slots, taps-1, C] fp32 with C = Cq+Ck+Cv; cs [P, rot_dims] fp32;
 // q_out [rows, Cq]; k_cache [NB, G, BS, kw], v_cache [NB, G, BS, vw] (empty
 // tensors when Ck == 0).
-void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
+bool conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
                       torch::Tensor v_cache, torch::Tensor proj,
                       torch::Tensor bias, torch::Tensor cw,
                       torch::Tensor state, torch::Tensor cs,
@@ -365,7 +379,8 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
                       torch::Tensor cu_rows, torch::Tensor state_slots,
                       torch::Tensor block_table, int64_t q_col, int64_t k_col,
                       int64_t v_col, int64_t Cq, int64_t Ck, int64_t Cv,
-                      int64_t map_dim, int64_t rot_dims) {
+                      int64_t map_dim, int64_t rot_dims,
+                      bool one_row_per_seq) {
   check_act(proj, "proj");
   check_f32(bias, "bias"); check_f32(cw, "cw"); check_f32(state, "state");
   check_f32(cs, "cs");
@@ -407,7 +422,8 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
     TORCH_CHECK(block_table.dim() == 2 && block_table.size(0) >= nseq);
     a.max_blocks = (int)block_table.size(1);
   }
-  if (rows == 0) return;
+  if (rows == 0) return false;
+  TORCH_CHECK(!one_row_per_seq || rows == nseq);
   auto stream = c10::hip::getCurrentHIPStream().stream();
   const bool kv = Ck > 0 || Cv > 0;
   const bool vec =
@@ -440,7 +456,7 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
     else KK_SLIDE(4);
 #undef KK_SLIDE
     HIP_CHECK_KERNEL();
-    return;
+    return false;
   }
   if (vec) {
     dim3 vgrid((unsigned)((rows + 7) / 8), (unsigned)((C / 8 + 31) / 32));
@@ -453,10 +469,11 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
           cw.data_ptr<float>(), state.data_ptr<float>(), cs.data_ptr<float>(),
           positions.data_ptr<int>(), row_seq.data_ptr<int>(),
           cu_rows.data_ptr<int>(), state_slots.data_ptr<int>(),
-          block_table.data_ptr<int>(), a, (int)rows);
+          block_table.data_ptr<int>(), a, (int)rows,
+          one_row_per_seq ? 1 : 0);
     });
     HIP_CHECK_KERNEL();
-    return;
+    return one_row_per_seq;
   }
   dim3 grid((unsigned)rows, (unsigned)((C + 255) / 256));
   KK_DISPATCH_ACT(proj, {
@@ -471,6 +488,7 @@ void conv_rope_append(torch::Tensor q_out, torch::Tensor k_cache,
         block_table.data_ptr<int>(), a);
   });
   HIP_CHECK_KERNEL();
+  return false;
 }
 
 void conv_state_update(torch::Tensor state, torch::Tensor proj,

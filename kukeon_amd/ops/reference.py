@@ -289,7 +289,8 @@ def _conv_cols(q_col, k_col, v_col, Cq, Ck, Cv):
 def conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw, state, cs,
                      positions, row_seq, cu_rows, state_slots, block_table,
                      q_col: int, k_col: int, v_col: int, Cq: int, Ck: int,
-                     Cv: int, map_dim: int, rot_dims: int) -> None:
+                     Cv: int, map_dim: int, rot_dims: int,
+                     one_row_per_seq: bool = False) -> bool:
     C = Cq + Ck + Cv
     taps = cw.shape[0]                     # cw: [taps, C]
     back = taps - 1
@@ -336,6 +337,7 @@ def conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw, state, cs,
                 blk = int(block_table[s, p // BS])
                 k_cache[blk, :, p % BS] = kk[i]
                 v_cache[blk, :, p % BS] = vv[i]
+    return False
 
 
 def conv_state_update(state, proj, bias, positions, cu_rows, state_slots,
