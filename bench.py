@@ -164,7 +164,8 @@ def main() -> None:
     else:
         device = "cpu"
 
-    cfg = MODEL_PRESETS[args.model]()
+    from kukeon_amd.models import registry
+    cfg = registry.preset(args.model)
     tp_size = world if args.model == "llama-3-70b" else 1
     # TP ranks share a sampling seed (identical draws, no collective needed)
     ecfg = EngineConfig(max_model_len=args.max_model_len,
@@ -184,12 +185,7 @@ def main() -> None:
     if use_ep:
         parallel.init_expert_parallel(world)
         ecfg.use_graphs = False  # all-to-all splits are data-dependent
-    if cfg.is_moe:
-        from kukeon_amd.models.mixtral import MixtralModel
-        model = MixtralModel(cfg, device=device)
-    else:
-        from kukeon_amd.models.llama import LlamaModel
-        model = LlamaModel(cfg, device=device)
+    model = registry.build_model(cfg, device)
 
     engine = LLMEngine(model, cfg, ecfg, device=device)
     tp = ecfg.tp_size

@@ -819,9 +819,12 @@ def daemon_stop(ctx):
 
 @daemon.command("recreate")
 @click.option("--model", default="llama-3-8b")
+@click.option("--model-dir", default="",
+              help="checkpoint folder (config.json + model.safetensors)")
+@click.option("--dtype", type=click.Choice(["", "bf16", "fp32"]), default="")
 @click.option("--gpus", type=int, default=1)
 @pass_ctx
-def daemon_recreate(ctx, model, gpus):
+def daemon_recreate(ctx, model, model_dir, dtype, gpus):
     """Re-provision the system modelhub cell (reference `kuke daemon
     recreate` re-provisions the containerized kukeond cell via
     ProvisionKukeondCell, controller.go:253-280 — here the system cell
@@ -833,7 +836,8 @@ def daemon_recreate(ctx, model, gpus):
                         naming.SYSTEM_STACK, "modelhub", force=True)
     except errors.NotFound:
         pass
-    doc = ctl.provision_modelhub_cell(model=model, gpus=gpus)
+    doc = ctl.provision_modelhub_cell(model=model, gpus=gpus,
+                                      model_dir=model_dir, dtype=dtype)
     click.echo(f"modelhub cell recreated: {doc.status.state}")
 
 

@@ -52,10 +52,36 @@ def build_model(cfg, device, **kw):
     return FAMILIES[family_of(cfg)](cfg, device, **kw)
 
 
+def _lipedra_preset(**kw):
+    def make():
+        from kukeon_amd.models.lipedra import lipedra_bench
+        return lipedra_bench(**kw)
+    return make
+
+
+# random-weight Lipedra stacks at Llama-3-8B layer sizes: 32 layers, every
+# second layer reading its predecessor's cache; and a small one for tests
+LIPEDRA_PRESETS = {
+    "lipedra-8b-like": _lipedra_preset(width=4096, layers=32, heads=32,
+                                       kv_heads=8, dim=64, vdim=128,
+                                       ff=14336, vocab=128256, share_every=2,
+                                       name="lipedra-8b-like"),
+    "tiny-lipedra": _lipedra_preset(width=256, layers=3, heads=4, kv_heads=2,
+                                    dim=16, vdim=32, ff=512, vocab=512,
+                                    share_every=3, name="tiny-lipedra"),
+}
+
+
+def preset_names():
+    return sorted(list(MODEL_PRESETS) + list(LIPEDRA_PRESETS))
+
+
 def preset(name: str):
+    if name in LIPEDRA_PRESETS:
+        return LIPEDRA_PRESETS[name]()
     if name not in MODEL_PRESETS:
         raise KeyError(f"unknown model preset {name!r}; known: "
-                       f"{sorted(MODEL_PRESETS)}")
+                       f"{preset_names()}")
     return MODEL_PRESETS[name]()
 
 

@@ -637,3 +637,42 @@ def case_tiles(device, dtype):
     got = run_schedule(eng, prompts, sched)
     for i in range(4):
         check(got[i], want[i], dtype, f"portions {i}")
+
+
+def _generate(eng, kv, prompt, n):
+    sp = SamplingParams(temperature=0.0, max_new_tokens=n)
+    eng.add_request(kv, prompt, sp)
+    out = []
+    while eng.has_work():
+        for o in eng.step():
+            out.extend(o.new_tokens)
+    return out
+
+
+def case_multi_turn(device, dtype):
+    """A session's second turn continues from its pages and state slot; an
+    idle session whose pages were taken away is rebuilt from its history."""
+    cfg = CONFIGS["mixed"]()
+    W = weights(cfg, 13)
+    mcfg = LipedraConfig.from_json(cfg)
+    model = LipedraModel(mcfg, device=device, dtype=dtype, tensors=W,
+                         max_position=128)
+    ecfg = EngineConfig(block_size=4, max_model_len=64, max_sessions=2,
+                        state_slots=2, num_kv_blocks=12, use_graphs=False,
+                        decode_microbatch=2)
+    eng = LLMEngine(model, mcfg, ecfg, device=device)
+    a, b = SequenceKV(4), SequenceKV(4)
+    p1, p2, p3 = tokens(cfg, 9, 60), tokens(cfg, 5, 61), tokens(cfg, 30, 62)
+    t1 = _generate(eng, a, p1, 4)
+    assert t1 == oracle.greedy(cfg, W, p1, 4)
+    t2 = _generate(eng, a, p2, 3)
+    assert t2 == oracle.greedy(cfg, W, p1 + t1 + p2, 3)
+    held = a.num_tokens
+    assert held > 0 and a.state_slot >= 0
+    # b needs more pages than are left: a's pages and slot are taken
+    tb = _generate(eng, b, p3, 4)
+    assert tb == oracle.greedy(cfg, W, p3, 4)
+    assert a.num_tokens == 0 and a.state_slot < 0 and a.history
+    eng.free_sequence(b)
+    t3 = _generate(eng, a, [7, 3], 3)
+    assert t3 == oracle.greedy(cfg, W, p1 + t1 + p2 + t2 + [7, 3], 3)

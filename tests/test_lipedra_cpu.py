@@ -59,6 +59,21 @@ def test_greedy_generation():
     cases.case_greedy(DEV, DT)
 
 
+def test_multi_turn_and_eviction():
+    cases.case_multi_turn(DEV, DT)
+
+
+def test_presets_and_registry():
+    from kukeon_amd.models import registry
+    assert "lipedra-8b-like" in registry.preset_names()
+    cfg = registry.preset("tiny-lipedra")
+    assert registry.family_of(cfg) == "lipedra"
+    model = registry.build_model(cfg, "cpu", dtype="fp32")
+    assert len(model.kv_specs()) == cfg.num_layers
+    assert model.kv_specs()[2].share_from == 1
+    assert registry.family_of(registry.preset("tiny-llama")) == "llama"
+
+
 def test_norm_op():
     cases.case_op_norm(DEV, DT)
 
