@@ -372,6 +372,7 @@ class LipedraLayer(nn.Module):
             return
         if (meta.mode == "prefill" and meta.max_rows >= 16 and
                 meta.chunk_lens is not None and
+                cat.stride(0) % 4 == 0 and      # 8-byte output stores
                 ops.diff_tiles_supported(q, m.dim, m.vdim)):
             hpg = m.heads // m.kv_heads
             hpw = 4 if hpg % 4 == 0 else 2 if hpg % 2 == 0 else 1

@@ -100,6 +100,15 @@ def _narrow():
 CONFIGS["narrow"] = _narrow
 
 
+# matrix-core sizes, but a feed-forward width that leaves the fused
+# [attention | feed-forward] rows unaligned
+CONFIGS["oddff"] = lambda: config([
+    layer(heads=4, kv_heads=2, dim=16, vdim=32, conv=2, rot_dims=8, ff=23),
+    layer(heads=4, kv_heads=2, dim=16, vdim=32, conv=2, rot_dims=8, ff=23,
+          kv_from=0),
+], width=32, vocab=41)
+
+
 def weights(cfg, seed=0):
     """Random checkpoint for a config dictionary, bf16 like a stored one."""
     g = torch.Generator().manual_seed(seed)
