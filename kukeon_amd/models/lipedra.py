@@ -140,13 +140,13 @@ def lipedra_bench(width=4096, layers=8, heads=32, kv_heads=8, dim=64,
     """A layer stack at real-model sizes (random weights) for throughput
     runs: every `share_every`-th layer reads its predecessor's cache."""
     rot = RotaryCfg(dims=dim, base=500000.0,
-                    scaling={"factor": 8.0, "original": 8192, "fast": 32.0,
-                             "slow": 1.0})
+                    scaling={"factor": 4.0, "original": 4096, "fast": 16.0,
+                             "slow": 2.0})
     ls = []
     for i in range(layers):
         shared = share_every > 1 and i % share_every == share_every - 1
         ls.append(LipedraLayerCfg(
-            DiffAttnCfg(heads, kv_heads, dim, vdim, conv=4, diff=0.3,
+            DiffAttnCfg(heads, kv_heads, dim, vdim, conv=4, diff=0.2,
                         scale=dim ** -0.5, rot=rot,
                         kv_from=(i - 1 if shared else None)),
             GluCfg(ff=ff, limit=7.0)))

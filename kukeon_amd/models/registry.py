@@ -66,8 +66,8 @@ LIPEDRA_PRESETS = {
                                        kv_heads=8, dim=64, vdim=128,
                                        ff=14336, vocab=128256, share_every=2,
                                        name="lipedra-8b-like"),
-    "tiny-lipedra": _lipedra_preset(width=256, layers=3, heads=4, kv_heads=2,
-                                    dim=16, vdim=32, ff=512, vocab=512,
+    "tiny-lipedra": _lipedra_preset(width=192, layers=3, heads=6, kv_heads=2,
+                                    dim=16, vdim=32, ff=320, vocab=384,
                                     share_every=3, name="tiny-lipedra"),
 }
 
