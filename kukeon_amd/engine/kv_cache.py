@@ -105,7 +105,10 @@ class LayerKVSpec:
 
 class LayeredKVCache:
     """Paged cache whose layers differ in shape (key rows wider than value
-    rows, per-layer head counts) and may share pages across layers.
+    rows, per-layer head counts) and may share pages across layers. A layer
+    whose spec is None keeps no pages at all (a recurrent mixer); a spec
+    with `v_width == 0` keeps one row per token (a latent cache from which
+    keys and values are both expanded).
 
     One allocator serves all layers: block id b names the page
     [b, kv_heads, block_size, width] in every layer's pool, so a sequence
@@ -122,7 +125,7 @@ class LayeredKVCache:
         self.k: List[torch.Tensor] = [None] * self.num_layers
         self.v: List[torch.Tensor] = [None] * self.num_layers
         for i, sp in enumerate(self.specs):
-            if sp.share_from is not None:
+            if sp is None or sp.share_from is not None:
                 continue
             # zeros: masked-out tail slots are never read as garbage
             self.k[i] = torch.zeros(num_blocks, sp.kv_heads, block_size,
@@ -130,10 +133,11 @@ class LayeredKVCache:
             self.v[i] = torch.zeros(num_blocks, sp.kv_heads, block_size,
                                     sp.v_width, dtype=dtype, device=device)
         for i, sp in enumerate(self.specs):
-            if sp.share_from is None:
+            if sp is None or sp.share_from is None:
                 continue
             j = sp.share_from
-            if not (0 <= j < i) or self.specs[j].share_from is not None:
+            if not (0 <= j < i) or self.specs[j] is None or \
+                    self.specs[j].share_from is not None:
                 raise ValueError(
                     f"layer {i} shares the cache of layer {j}, which must be "
                     "an earlier layer with pages of its own")
@@ -150,20 +154,24 @@ class LayeredKVCache:
     def nbytes(self) -> int:
         return sum(self.k[i].nbytes + self.v[i].nbytes
                    for i, sp in enumerate(self.specs)
-                   if sp.share_from is None)
+                   if sp is not None and sp.share_from is None)
 
     @staticmethod
     def blocks_from_bytes(free_bytes: int, specs: Sequence[LayerKVSpec],
                           block_size: int, dtype_bytes: int = 2) -> int:
         per_block = sum(sp.kv_heads * block_size * (sp.k_width + sp.v_width)
-                        for sp in specs if sp.share_from is None) * dtype_bytes
+                        for sp in specs
+                        if sp is not None and sp.share_from is None) \
+            * dtype_bytes
         return max(1, free_bytes // max(1, per_block))
 
 
 class StatePool:
     """Fixed-size slots of per-sequence carried state (tails of short
     convolutions, recurrent state): one fp32 tensor [slots, *shape] per
-    layer that carries state, None for the others. A sequence holds one
+    layer that carries state, None for the others; a layer that carries
+    several pieces (a convolution tail AND a recurrent state) gives a list
+    of shapes and gets a tuple of tensors. A sequence holds one
     slot index for all layers; a slot's content is only meaningful to the
     sequence that wrote it, and a sequence that starts at position 0 never
     reads what the slot held before."""
@@ -171,10 +179,15 @@ class StatePool:
     def __init__(self, layer_shapes: Sequence[Optional[Tuple[int, ...]]],
                  num_slots: int, device, dtype=torch.float32):
         self.num_slots = num_slots
-        self.layers: List[Optional[torch.Tensor]] = [
-            None if shp is None else
-            torch.zeros((num_slots,) + tuple(shp), dtype=dtype, device=device)
-            for shp in layer_shapes]
+        def make(shp):
+            if shp is None:
+                return None
+            if len(shp) and isinstance(shp[0], (tuple, list)):
+                return tuple(make(one) for one in shp)
+            return torch.zeros((num_slots,) + tuple(shp), dtype=dtype,
+                               device=device)
+
+        self.layers: list = [make(shp) for shp in layer_shapes]
         self._free: List[int] = list(range(num_slots - 1, -1, -1))
 
     @property

@@ -1,0 +1,235 @@
+"""Sequence mixers that carry their own kind of memory: a selective
+state-space mixer (fixed-size recurrent state per sequence) and a latent
+attention mixer (one low-rank row per token in the paged cache). Both take
+the normed layer input [T, W] of a packed batch plus the engine's row maps
+and return the mixer output [T, W]; all sizes and constants are arguments,
+so any model family can stack them.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Optional
+
+import torch
+import torch.nn as nn
+
+from kukeon_amd import ops
+from kukeon_amd.engine.kv_cache import LayerKVSpec
+
+
+def _pad8(n: int) -> int:
+    return (n + 7) // 8 * 8
+
+
+def fuse_rows(segs, width: int, dtype, device):
+    """Stack projection weights [rows_i, width] into one matrix whose
+    segments each start on a multiple of 8 output columns.
+    -> ({name: first column}, parameter)."""
+    col, rows, at = {}, [], 0
+    for name, wt in segs:
+        col[name] = at
+        n = wt.shape[0]
+        rows.append(wt.to(device=device, dtype=dtype))
+        pad = _pad8(n) - n
+        if pad:
+            rows.append(torch.zeros(pad, width, dtype=dtype, device=device))
+        at += _pad8(n)
+    return col, nn.Parameter(torch.cat(rows, 0).contiguous(),
+                             requires_grad=False)
+
+
+# ---------------------------------------------------------------------------
+@dataclass
+class StateSpaceCfg:
+    heads: int
+    vdim: int                # channels per head
+    state: int               # rows of a head's state matrix
+    groups: int              # B/C groups; head h reads group h // (heads/groups)
+    conv: int                # taps of the short convolution
+    norm_groups: int         # parts of the gated output normed separately
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+
+class StateSpaceMixer(nn.Module):
+    """Selective state-space mixer (the recurrent form of state-space
+    duality). The input projection yields [z | x | B | C | dt]; x, B and C
+    pass a short causal convolution and silu; per head
+    S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x with
+    dt = softplus(dt + dt_bias); y is gated by silu(z), normed in
+    `norm_groups` parts and projected out. The state matrix and the last
+    taps-1 convolution inputs live in the engine's state slots (fp32).
+
+    Tensors (prefix p): in [2*inner + 2*G*N + H, W], conv [C, taps],
+    conv.b [C], dt_bias, A_log, D [H], norm [inner], o [W, inner]."""
+
+    def __init__(self, m: StateSpaceCfg, width: int, eps: float,
+                 t: Dict[str, torch.Tensor], p: str, device, dtype):
+        super().__init__()
+        if m.heads % m.groups:
+            raise ValueError(f"{p}: heads not a multiple of groups")
+        if m.inner % m.norm_groups:
+            raise ValueError(f"{p}: inner size not divisible by norm_groups")
+        self.m = m
+        self.eps = eps
+        C = m.conv_channels
+        w_in = t[p + "in"]
+        if w_in.shape[0] != 2 * m.inner + 2 * m.groups * m.state + m.heads:
+            raise ValueError(f"{p}in: rows do not fit the mixer's sizes")
+        self.w_in = nn.Parameter(w_in.to(device=device, dtype=dtype)
+                                 .contiguous(), requires_grad=False)
+        cw = t[p + "conv"]
+        if tuple(cw.shape) != (C, m.conv):
+            raise ValueError(f"{p}conv: shape {tuple(cw.shape)}")
+        f32 = dict(device=device, dtype=torch.float32)
+        self.conv_w = cw.to(**f32).t().contiguous()          # [taps, C]
+        self.conv_b = t[p + "conv.b"].to(**f32).contiguous()
+        self.zero_b = torch.zeros(C, **f32)
+        self.dt_bias = t[p + "dt_bias"].to(**f32).contiguous()
+        self.rate = torch.exp(t[p + "A_log"].to(**f32)).contiguous()
+        self.skip = t[p + "D"].to(**f32).contiguous()
+        self.norm_w = t[p + "norm"].to(**f32).contiguous()
+        self.w_o = nn.Parameter(t[p + "o"].to(device=device, dtype=dtype)
+                                .contiguous(), requires_grad=False)
+
+    @staticmethod
+    def tensor_shapes(m: StateSpaceCfg, width: int) -> Dict[str, tuple]:
+        C = m.conv_channels
+        return {"in": (2 * m.inner + 2 * m.groups * m.state + m.heads, width),
+                "conv": (C, m.conv), "conv.b": (C,), "dt_bias": (m.heads,),
+                "A_log": (m.heads,), "D": (m.heads,), "norm": (m.inner,),
+                "o": (width, m.inner)}
+
+    def kv_spec(self) -> Optional[LayerKVSpec]:
+        return None
+
+    def state_shape(self):
+        m = self.m
+        return [(m.conv - 1, m.conv_channels), (m.heads, m.state, m.vdim)]
+
+    def forward(self, h: torch.Tensor, cache, state, meta) -> torch.Tensor:
+        m = self.m
+        T = h.shape[0]
+        conv_state, ssm_state = state
+        proj = ops.linear(h, self.w_in)
+        inner, C = m.inner, m.conv_channels
+        xbc = torch.empty(T, C, dtype=h.dtype, device=h.device)
+        ops.conv_act(xbc, proj, inner, self.conv_w, self.conv_b, conv_state,
+                     meta.positions, meta.row_seq, meta.cu_rows,
+                     meta.state_slots, 1)
+        ops.conv_tail_update(conv_state, proj, inner, self.zero_b,
+                             meta.positions, meta.cu_rows, meta.state_slots)
+        y = torch.empty(T, inner, dtype=torch.float32, device=h.device)
+        ops.ssm_scan(y, xbc, proj[:, inner + C:inner + C + m.heads],
+                     self.dt_bias, self.rate, self.skip, ssm_state,
+                     meta.positions, meta.cu_rows, meta.state_slots,
+                     m.heads, m.vdim, m.state, m.groups)
+        g = torch.empty(T, inner, dtype=h.dtype, device=h.device)
+        ops.gated_group_rmsnorm(g, y, proj[:, :inner], self.norm_w,
+                                m.norm_groups, self.eps)
+        return ops.linear(g, self.w_o)
+
+
+# ---------------------------------------------------------------------------
+@dataclass
+class LatentAttnCfg:
+    heads: int
+    dim: int                 # unrotated query/key entries per head
+    rot_dim: int             # rotated entries per head (one shared key part)
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    window: int              # position i sees i-window+1 .. i (0: all)
+    rot_dims: int            # leading entries of the rotated part that turn
+    rot_base: float
+
+
+class LatentAttention(nn.Module):
+    """Attention over a low-rank latent. Per token the cache holds ONE row
+    [c | k_rot]: the normed latent c (kv_rank) from which every head's
+    unrotated keys (W_uk c) and values (W_uv c) derive, and one rotated key
+    part shared by all heads. The products with W_uk and W_uv are moved to
+    the query and the output side,
+
+        score_h(i, j) = ((W_uk_h^T q_h)(i) . c(j) + rot(q_rot_h)(i) . k_rot(j)) scale
+        out_h(i)      = W_uv_h  sum_j softmax_j(score_h)(i, j) c(j)
+
+    so the kernel reads each cache row once for all heads. Queries pass
+    their own normed latent (q_rank). A sliding window bounds the keys, and
+    every head's output is scaled by sigmoid of a gate projected from the
+    mixer's input.
+
+    Tensors (prefix p): dq [q_rank, W], dq.norm, uq [H*(dim+rot_dim), q_rank],
+    dkv [kv_rank+rot_dim, W], dkv.norm, uk [H*dim, kv_rank],
+    uv [H*vdim, kv_rank], g [H, W], o [W, H*vdim]."""
+
+    def __init__(self, m: LatentAttnCfg, width: int, eps: float,
+                 t: Dict[str, torch.Tensor], p: str, device, dtype):
+        super().__init__()
+        if m.rot_dims % 2 or m.rot_dims > m.rot_dim:
+            raise ValueError(f"{p}: bad rotary dims")
+        self.m = m
+        self.eps = eps
+        self.col, self.w_down = fuse_rows(
+            [("q", t[p + "dq"]), ("kv", t[p + "dkv"]), ("g", t[p + "g"])],
+            width, dtype, device)
+        f32 = dict(device=device, dtype=torch.float32)
+        self.q_norm = t[p + "dq.norm"].to(**f32).contiguous()
+        self.kv_norm = t[p + "dkv.norm"].to(**f32).contiguous()
+        dev = dict(device=device, dtype=dtype)
+        self.w_uq = nn.Parameter(t[p + "uq"].to(**dev).contiguous(),
+                                 requires_grad=False)
+        H, R = m.heads, m.kv_rank
+        # [H, dim, R]: q_abs_h = q_h W_uk_h;  [H, R, vdim]: o_h = l_h W_uv_h^T
+        self.w_uk = nn.Parameter(t[p + "uk"].to(**dev).view(H, m.dim, R)
+                                 .contiguous(), requires_grad=False)
+        self.w_uv = nn.Parameter(t[p + "uv"].to(**dev).view(H, m.vdim, R)
+                                 .transpose(1, 2).contiguous(),
+                                 requires_grad=False)
+        self.w_o = nn.Parameter(t[p + "o"].to(**dev).contiguous(),
+                                requires_grad=False)
+        self.cs = None       # angle table [positions, rot_dims], set by the model
+
+    @staticmethod
+    def tensor_shapes(m: LatentAttnCfg, width: int) -> Dict[str, tuple]:
+        H = m.heads
+        return {"dq": (m.q_rank, width), "dq.norm": (m.q_rank,),
+                "uq": (H * (m.dim + m.rot_dim), m.q_rank),
+                "dkv": (m.kv_rank + m.rot_dim, width),
+                "dkv.norm": (m.kv_rank,), "uk": (H * m.dim, m.kv_rank),
+                "uv": (H * m.vdim, m.kv_rank), "g": (H, width),
+                "o": (width, H * m.vdim)}
+
+    def kv_spec(self) -> Optional[LayerKVSpec]:
+        return LayerKVSpec(1, self.m.kv_rank + self.m.rot_dim, 0)
+
+    def state_shape(self):
+        return None
+
+    def forward(self, h: torch.Tensor, cache, state, meta) -> torch.Tensor:
+        m = self.m
+        T = h.shape[0]
+        H, R = m.heads, m.kv_rank
+        proj = ops.linear(h, self.w_down)
+        cq = torch.empty(T, m.q_rank, dtype=h.dtype, device=h.device)
+        ops.latent_kv_append(cq, cache, proj, self.col["q"], self.col["kv"],
+                             self.q_norm, self.kv_norm, self.eps, self.cs,
+                             meta.positions, meta.row_seq, meta.block_table)
+        q = ops.linear(cq, self.w_uq)                  # [T, H*(dim+rot)]
+        q_n = q.view(T, H, m.dim + m.rot_dim)[:, :, :m.dim].transpose(0, 1)
+        q_abs = torch.bmm(q_n, self.w_uk)              # [H, T, R]
+        lat = torch.empty(H, T, R, dtype=h.dtype, device=h.device)
+        ops.latent_attention(lat, q_abs, q, cache, self.cs, meta.positions,
+                             meta.row_seq, meta.block_table, H, m.dim,
+                             m.rot_dim, m.window, m.scale)
+        o = torch.bmm(lat, self.w_uv)                  # [H, T, vdim]
+        og = torch.empty(T, H * m.vdim, dtype=h.dtype, device=h.device)
+        ops.head_gate(og, o, proj[:, self.col["g"]: self.col["g"] + H])
+        return ops.linear(og, self.w_o)

@@ -27,16 +27,33 @@ def _lipedra(cfg, device, **kw):
     return LipedraModel(cfg, device=device, **kw)
 
 
+def _rasesun(cfg, device, **kw):
+    from kukeon_amd.models.rasesun import RasesunModel
+    return RasesunModel(cfg, device=device, **kw)
+
+
 # family -> constructor(cfg, device, **kw)
 FAMILIES: Dict[str, Callable] = {
     "llama": _llama,
     "mixtral": _mixtral,
     "lipedra": _lipedra,
+    "rasesun": _rasesun,
 }
 
 # config.json "architecture" -> family
 ARCHITECTURES: Dict[str, str] = {
     "Lipedra": "lipedra",
+    "Rasesun": "rasesun",
+}
+
+
+# family -> kernel groups its forward pass needs on a GPU (the sampler and
+# the weight-streaming GEMMs of the "core" group are optional for these)
+OP_GROUPS: Dict[str, tuple] = {
+    "llama": ("core",),
+    "mixtral": ("core",),
+    "lipedra": ("mix",),
+    "rasesun": ("recur",),
 }
 
 
@@ -96,5 +113,9 @@ def load_checkpoint(model_dir: str, device, dtype: str = "bf16"):
     if fam == "lipedra":
         from kukeon_amd.models.lipedra import LipedraModel
         return LipedraModel.from_checkpoint(model_dir, device=device,
+                                            dtype=dtype)
+    if fam == "rasesun":
+        from kukeon_amd.models.rasesun import RasesunModel
+        return RasesunModel.from_checkpoint(model_dir, device=device,
                                             dtype=dtype)
     raise ValueError(f"family {fam} has no checkpoint loader")

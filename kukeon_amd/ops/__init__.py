@@ -27,6 +27,14 @@ except Exception as e:  # pragma: no cover
     _MIX_IMPORT_ERROR = e
 
 
+_C_recur = None
+_RECUR_IMPORT_ERROR: Exception | None = None
+try:
+    from kukeon_amd import _C_recur  # type: ignore
+except Exception as e:  # pragma: no cover
+    _RECUR_IMPORT_ERROR = e
+
+
 def native_available() -> bool:
     return _C is not None
 
@@ -54,6 +62,31 @@ def _mix(t: torch.Tensor):
             "was called on a CUDA device. Run `python -m kukeon_amd.ops.build "
             f"mix` (import error: {_MIX_IMPORT_ERROR})")
     return _C_mix
+
+
+def recur_available() -> bool:
+    return _C_recur is not None
+
+
+def _recur(t: torch.Tensor):
+    """Kernel group of the recurrent and latent mixers: native on a GPU
+    tensor (an error if the module is not built), fp32 references on CPU."""
+    global _C_recur, _RECUR_IMPORT_ERROR
+    if not t.is_cuda:
+        return reference
+    if _C_recur is None:
+        try:
+            import importlib
+            _C_recur = importlib.import_module("kukeon_amd._C_recur")
+        except Exception as e:
+            _RECUR_IMPORT_ERROR = e
+    if _C_recur is None:
+        raise RuntimeError(
+            "kukeon_amd._C_recur (gfx950 HIP extension) is not built but an "
+            "op was called on a CUDA device. Run `python -m "
+            f"kukeon_amd.ops.build recur` (import error: "
+            f"{_RECUR_IMPORT_ERROR})")
+    return _C_recur
 
 
 def _native():
@@ -430,3 +463,73 @@ def diff_attention_decode(out, q, k_cache, v_cache, gate, positions, row_seq,
                                   gate if gate is not None else _e(q),
                                   positions, row_seq, block_table, part_o,
                                   part_ml, H, scale, lam, eps, out_scale)
+
+
+# ---- recurrent / latent group ----------------------------------------------
+def norm_only(x, w, eps: float, out) -> None:
+    """out = rmsnorm(x) * w over the fp32 residual stream (x unchanged)."""
+    _recur(x).residual_add_rmsnorm(x, _e(out), _e(x), w, 0.0, eps, out)
+
+
+def postnorm_residual_rmsnorm(x, y, post_w, w, eps: float, out) -> None:
+    """Sandwich norms in one pass over a row: x (fp32, in place) +=
+    rmsnorm(y) * post_w, then out = rmsnorm(x) * w."""
+    _recur(x).postnorm_residual_rmsnorm(x, y, post_w, w, eps, out)
+
+
+def conv_act(out, proj, col0: int, cw, bias, state, positions, row_seq,
+             cu_rows, state_slots, act: int = 1) -> None:
+    """Short causal convolution per channel over proj[:, col0:col0+C] with
+    carried taps, bias after the sum, then the activation (1: silu, 0:
+    none). Does not touch the state; conv_tail_update shifts it."""
+    _recur(proj).conv_act(out, proj, col0, cw, bias, state, positions,
+                          row_seq, cu_rows, state_slots, act)
+
+
+def conv_tail_update(state, proj, col0: int, zero_bias, positions, cu_rows,
+                     state_slots) -> None:
+    """Shift a portion's last inputs into the convolution state slots."""
+    C = state.shape[2]
+    _recur(proj).conv_state_update(state, proj, zero_bias, positions,
+                                   cu_rows, state_slots, col0, 0, 0, C, 0, 0)
+
+
+def ssm_scan(y, xbc, dt, dt_bias, rate, skip, state, positions, cu_rows,
+             state_slots, H: int, P: int, N: int, G: int) -> None:
+    _recur(xbc).ssm_scan(y, xbc, dt, dt_bias, rate, skip, state, positions,
+                         cu_rows, state_slots, H, P, N, G)
+
+
+def gated_group_rmsnorm(out, y, z, w, groups: int, eps: float) -> None:
+    _recur(out).gated_group_rmsnorm(out, y, z, w, groups, eps)
+
+
+def latent_kv_append(cq_out, cache, proj, q_col: int, kv_col: int, wq, wkv,
+                     eps: float, cs, positions, row_seq,
+                     block_table) -> None:
+    _recur(proj).latent_kv_append(cq_out, cache, proj, q_col, kv_col, wq,
+                                  wkv, eps, cs, positions, row_seq,
+                                  block_table)
+
+
+def latent_attention(out, q_abs, q, cache, cs, positions, row_seq,
+                     block_table, H: int, dn: int, dr: int, window: int,
+                     scale: float) -> None:
+    _recur(q).latent_attention(out, q_abs, q, cache, cs, positions, row_seq,
+                               block_table, H, dn, dr, window, scale)
+
+
+def head_gate(out, o, gate) -> None:
+    _recur(out).head_gate(out, o, gate)
+
+
+def xielu(out, z, ap: float, aq: float) -> None:
+    _recur(out).xielu(out, z, ap, aq)
+
+
+def table_moe(out, h, ids, table, w_up, w_down) -> None:
+    _recur(h).table_moe(out, h, ids, table, w_up, w_down)
+
+
+def softcap_(logits, cap: float) -> None:
+    _recur(logits).softcap_(logits, cap)

@@ -33,6 +33,20 @@ MIX_SOURCES = [
     "bindings_mix.cpp",
 ]
 
+#   recur -> kukeon_amd/_C_recur.so (sandwich norms, convolution with
+#                                  activation, state-space scan, latent
+#                                  attention, table-routed experts)
+RECUR_SOURCES = [
+    "resid_norm.hip",
+    "short_conv.hip",
+    "conv_act.hip",
+    "ssm_scan.hip",
+    "recur_elem.hip",
+    "latent_attn.hip",
+    "table_moe.hip",
+    "bindings_recur.cpp",
+]
+
 SOURCES = [
     "rmsnorm.hip",
     "activation.hip",
@@ -63,6 +77,7 @@ def _run(cmd: list[str]) -> None:
 GROUPS = {
     "core": ("_C", SOURCES),
     "mix": ("_C_mix", MIX_SOURCES),
+    "recur": ("_C_recur", RECUR_SOURCES),
 }
 
 

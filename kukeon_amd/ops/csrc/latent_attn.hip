@@ -1,0 +1,306 @@
+// Latent attention: per token the paged cache holds ONE row
+// [c (R entries) | k_rot (dr entries)] shared by all heads.
+//
+// latent_kv_append   norms the query latent and the key/value latent of
+//                    every row, rotates the shared key part and writes the
+//                    cache row.
+// latent_attention   for every (row, head): scores over the last `window`
+//                    positions, q_abs . c + rot(q_rot) . k_rot, softmax,
+//                    and the weighted sum of the latents c. The products
+//                    with the per-head key and value expansions live
+//                    outside, on the query and output side.
+//
+// Everything is accumulated in fp32. A row walks its keys oldest first in
+// chunks counted from the first visible key, so its result depends only on
+// its own position and window.
+#include "elem.h"
+
+namespace kukeon {
+
+// One block per row. cs [positions, dims] = [cos_0.. | sin_0..]; pairs
+// (2i, 2i+1) of the first `dims` entries of the rotated part turn.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_kv_append_kernel(
+    T* __restrict__ cq_out, T* __restrict__ cache, const T* __restrict__ proj,
+    long ldp, long q_col, long kv_col, const float* __restrict__ wq,
+    const float* __restrict__ wkv, float eps, const float* __restrict__ cs,
+    int cs_rows, int dims, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ block_table,
+    int max_blocks, int Rq, int R, int dr, int BS) {
+  __shared__ float red[32];
+  const long r = blockIdx.x;
+  const int p = positions[r];
+  if (p < 0) return;
+  const T* row = proj + r * ldp;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < Rq; i += blockDim.x) {
+    const float v = ldf(row + q_col + i);
+    sq += v * v;
+  }
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    const float v = ldf(row + kv_col + i);
+    sk += v * v;
+  }
+  const float2 tot = block_sum2(sq, sk, red);
+  const float rq = 1.0f / sqrtf(tot.x / (float)Rq + eps);
+  const float rk = 1.0f / sqrtf(tot.y / (float)R + eps);
+  for (int i = threadIdx.x; i < Rq; i += blockDim.x)
+    stf(cq_out + r * (long)Rq + i, ldf(row + q_col + i) * rq * wq[i]);
+  const int s = row_seq[r];
+  const long blk = block_table[(long)s * max_blocks + p / BS];
+  T* crow = cache + (blk * BS + p % BS) * (long)(R + dr);
+  for (int i = threadIdx.x; i < R; i += blockDim.x)
+    stf(crow + i, ldf(row + kv_col + i) * rk * wkv[i]);
+  const int pp = p < cs_rows ? p : cs_rows - 1;
+  const float* ang = cs + (long)pp * dims;
+  const int half = dims / 2;
+  for (int i = threadIdx.x; i < dr; i += blockDim.x) {
+    const float v = ldf(row + kv_col + R + i);
+    float o = v;
+    if (i < dims) {
+      const int pr = i >> 1;
+      const float other = ldf(row + kv_col + R + (i ^ 1));
+      const float c = ang[pr], sn = ang[half + pr];
+      o = (i & 1) ? fmaf(v, c, other * sn) : fmaf(v, c, -other * sn);
+    }
+    stf(crow + R + i, o);
+  }
+}
+
+void latent_kv_append(torch::Tensor cq_out, torch::Tensor cache,
+                      torch::Tensor proj, int64_t q_col, int64_t kv_col,
+                      torch::Tensor wq, torch::Tensor wkv, double eps,
+                      torch::Tensor cs, torch::Tensor positions,
+                      torch::Tensor row_seq, torch::Tensor block_table) {
+  check_act(proj, "proj");
+  check_f32(wq, "wq"); check_f32(wkv, "wkv"); check_f32(cs, "cs");
+  check_i32(positions, "positions"); check_i32(row_seq, "row_seq");
+  check_i32(block_table, "block_table");
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1);
+  const long rows = proj.size(0);
+  const int Rq = (int)wq.numel(), R = (int)wkv.numel();
+  TORCH_CHECK(cache.dim() == 4 && cache.is_contiguous() && cache.size(1) == 1 &&
+              cache.scalar_type() == proj.scalar_type());
+  const int BS = (int)cache.size(2);
+  const int dr = (int)cache.size(3) - R;
+  TORCH_CHECK(dr >= 0);
+  TORCH_CHECK(cs.dim() == 2 && cs.size(0) >= 1);
+  const int dims = (int)cs.size(1);
+  TORCH_CHECK(dims % 2 == 0 && dims <= dr);
+  TORCH_CHECK(q_col >= 0 && q_col + Rq <= proj.size(1) && kv_col >= 0 &&
+              kv_col + R + dr <= proj.size(1));
+  TORCH_CHECK(cq_out.dim() == 2 && cq_out.is_contiguous() &&
+              cq_out.size(0) == rows && cq_out.size(1) == Rq &&
+              cq_out.scalar_type() == proj.scalar_type());
+  TORCH_CHECK(positions.numel() == rows && row_seq.numel() == rows);
+  TORCH_CHECK(block_table.dim() == 2);
+  if (rows == 0) return;
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+#define KK_ARGS reinterpret_cast<T*>(out.data_ptr()),                        \
+        reinterpret_cast<const T*>(q_abs.data_ptr()),                        \
+        reinterpret_cast<const T*>(q.data_ptr()), (long)q.stride(0),         \
+        reinterpret_cast<const T*>(cache.data_ptr()), cs.data_ptr<float>(),  \
+        (int)cs.size(0), (int)cs.size(1), positions.data_ptr<int>(),         \
+        row_seq.data_ptr<int>(), block_table.data_ptr<int>(),                \
+        (int)block_table.size(1), rows, (int)H, (int)dn, (int)dr, R,         \
+        (int)cache.size(2), (int)window, (float)scale
+  KK_DISPATCH_ACT(proj, {
+    latent_kv_append_kernel<T><<<dim3((unsigned)rows), 256, 0, stream>>>(
+        reinterpret_cast<T*>(cq_out.data_ptr()),
+        reinterpret_cast<T*>(cache.data_ptr()),
+        reinterpret_cast<const T*>(proj.data_ptr()), (long)proj.stride(0),
+        (long)q_col, (long)kv_col, wq.data_ptr<float>(), wkv.data_ptr<float>(),
+        (float)eps, cs.data_ptr<float>(), (int)cs.size(0), dims,
+        positions.data_ptr<int>(), row_seq.data_ptr<int>(),
+        block_table.data_ptr<int>(), (int)block_table.size(1), Rq, R, dr, BS);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------------------------------------
+// Row-wise attention, any sizes, both formats. Block = (row, HB heads), 256
+// threads. Keys are taken 256 at a time: thread j scores key j for the HB
+// heads (the query vectors sit in LDS as fp32 and are read as broadcasts),
+// the block agrees on the running maximum and sum, then thread d sums the
+// weighted latents for output entries d, d+256, ...
+#define LAT_HB 4
+#define LAT_CH 256
+
+template <typename T, int ND>
+__global__ __launch_bounds__(256) void latent_attention_kernel(
+    T* __restrict__ out, const T* __restrict__ q_abs, const T* __restrict__ q,
+    long ldq, const T* __restrict__ cache, const float* __restrict__ cs,
+    int cs_rows, int dims, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ block_table,
+    int max_blocks, long rows, int H, int dn, int dr, int R, int BS,
+    int window, float scale) {
+  extern __shared__ float sm[];
+  const int KW = R + dr;
+  float* sq = sm;                          // [HB][KW] query (latent | rot)
+  float* sc = sq + LAT_HB * KW;            // [HB][CH] scores / weights
+  __shared__ float red[32];
+  __shared__ long srow[LAT_CH];            // first element of each key's row
+  const long r = blockIdx.x;
+  const int h0 = blockIdx.y * LAT_HB;
+  const int tid = threadIdx.x;
+  const int p = positions[r];
+  if (p < 0) {
+    for (int hb = 0; hb < LAT_HB && h0 + hb < H; ++hb)
+      for (int d = tid; d < R; d += blockDim.x)
+        stf(out + ((long)(h0 + hb) * rows + r) * R + d, 0.f);
+    return;
+  }
+  const int s = row_seq[r];
+  const int pp = p < cs_rows ? p : cs_rows - 1;
+  const float* ang = cs + (long)pp * dims;
+  const int half = dims / 2;
+  for (int i = tid; i < LAT_HB * KW; i += blockDim.x) {
+    const int hb = i / KW, d = i - hb * KW;
+    const int h = h0 + hb;
+    float v = 0.f;
+    if (h < H) {
+      if (d < R) {
+        v = ldf(q_abs + ((long)h * rows + r) * R + d);
+      } else {
+        const int e = d - R;
+        const T* qr = q + r * ldq + (long)h * (dn + dr) + dn;
+        v = ldf(qr + e);
+        if (e < dims) {
+          const float other = ldf(qr + (e ^ 1));
+          const float c = ang[e >> 1], sn = ang[half + (e >> 1)];
+          v = (e & 1) ? fmaf(v, c, other * sn) : fmaf(v, c, -other * sn);
+        }
+      }
+    }
+    sq[i] = v;
+  }
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int nkeys = p - lo + 1;
+  float m[LAT_HB], l[LAT_HB], acc[LAT_HB][ND];
+#pragma unroll
+  for (int hb = 0; hb < LAT_HB; ++hb) {
+    m[hb] = -INFINITY;
+    l[hb] = 0.f;
+#pragma unroll
+    for (int k = 0; k < ND; ++k) acc[hb][k] = 0.f;
+  }
+  const int* bt = block_table + (long)s * max_blocks;
+  for (int c0 = 0; c0 < nkeys; c0 += LAT_CH) {
+    const int cn = min(LAT_CH, nkeys - c0);
+    __syncthreads();                       // sq ready / previous chunk done
+    float sv[LAT_HB];
+#pragma unroll
+    for (int hb = 0; hb < LAT_HB; ++hb) sv[hb] = -INFINITY;
+    if (tid < cn) {
+      const int j = lo + c0 + tid;
+      const long base = ((long)bt[j / BS] * BS + j % BS) * KW;
+      srow[tid] = base;
+      const T* kr = cache + base;
+      float a[LAT_HB];
+#pragma unroll
+      for (int hb = 0; hb < LAT_HB; ++hb) a[hb] = 0.f;
+      for (int d = 0; d < KW; ++d) {
+        const float kv = ldf(kr + d);
+#pragma unroll
+        for (int hb = 0; hb < LAT_HB; ++hb)
+          a[hb] = fmaf(sq[hb * KW + d], kv, a[hb]);
+      }
+#pragma unroll
+      for (int hb = 0; hb < LAT_HB; ++hb) sv[hb] = a[hb] * scale;
+    }
+    float alpha[LAT_HB];
+#pragma unroll
+    for (int hb = 0; hb < LAT_HB; hb += 2) {
+      const float2 mx = block_max2(sv[hb], sv[hb + 1], red);
+      const float m0 = fmaxf(m[hb], mx.x), m1 = fmaxf(m[hb + 1], mx.y);
+      alpha[hb] = __expf(m[hb] - m0);       // first chunk: exp(-inf) = 0
+      alpha[hb + 1] = __expf(m[hb + 1] - m1);
+      m[hb] = m0;
+      m[hb + 1] = m1;
+      const float w0 = tid < cn ? __expf(sv[hb] - m0) : 0.f;
+      const float w1 = tid < cn ? __expf(sv[hb + 1] - m1) : 0.f;
+      sc[hb * LAT_CH + tid] = w0;
+      sc[(hb + 1) * LAT_CH + tid] = w1;
+      const float2 su = block_sum2(w0, w1, red);
+      l[hb] = l[hb] * alpha[hb] + su.x;
+      l[hb + 1] = l[hb + 1] * alpha[hb + 1] + su.y;
+    }
+    // block_sum2 ends with a barrier: sc and srow are visible
+#pragma unroll
+    for (int hb = 0; hb < LAT_HB; ++hb)
+#pragma unroll
+      for (int k = 0; k < ND; ++k) acc[hb][k] *= alpha[hb];
+    for (int jj = 0; jj < cn; ++jj) {
+      const T* kr = cache + srow[jj];
+#pragma unroll
+      for (int k = 0; k < ND; ++k) {
+        const int d = tid + k * 256;
+        if (d < R) {
+          const float cv = ldf(kr + d);
+#pragma unroll
+          for (int hb = 0; hb < LAT_HB; ++hb)
+            acc[hb][k] = fmaf(sc[hb * LAT_CH + jj], cv, acc[hb][k]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int hb = 0; hb < LAT_HB; ++hb) {
+    const int h = h0 + hb;
+    if (h >= H) break;
+    const float inv = 1.0f / l[hb];
+#pragma unroll
+    for (int k = 0; k < ND; ++k) {
+      const int d = tid + k * 256;
+      if (d < R) stf(out + ((long)h * rows + r) * R + d, acc[hb][k] * inv);
+    }
+  }
+}
+
+// out, q_abs [H, rows, R] contiguous; q [rows, >= H*(dn+dr)] (stride(1) ==
+// 1); cache [blocks, 1, BS, R+dr]; cs [positions, dims] fp32.
+void latent_attention(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q,
+                      torch::Tensor cache, torch::Tensor cs,
+                      torch::Tensor positions, torch::Tensor row_seq,
+                      torch::Tensor block_table, int64_t H, int64_t dn,
+                      int64_t dr, int64_t window, double scale) {
+  check_act(q, "q"); check_act(q_abs, "q_abs"); check_act(out, "out");
+  check_f32(cs, "cs");
+  check_i32(positions, "positions"); check_i32(row_seq, "row_seq");
+  check_i32(block_table, "block_table");
+  TORCH_CHECK(q_abs.dim() == 3 && q_abs.is_contiguous() && out.dim() == 3 &&
+              out.is_contiguous());
+  const long rows = q.size(0);
+  const int R = (int)q_abs.size(2);
+  TORCH_CHECK(q_abs.size(0) == H && q_abs.size(1) == rows &&
+              out.size(0) == H && out.size(1) == rows && out.size(2) == R);
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 &&
+              q.size(1) >= H * (dn + dr));
+  TORCH_CHECK(cache.dim() == 4 && cache.is_contiguous() && cache.size(1) == 1 &&
+              cache.size(3) == R + dr);
+  TORCH_CHECK(q.scalar_type() == cache.scalar_type() &&
+              q_abs.scalar_type() == cache.scalar_type() &&
+              out.scalar_type() == cache.scalar_type());
+  TORCH_CHECK(cs.dim() == 2 && cs.size(0) >= 1 && cs.size(1) % 2 == 0 &&
+              cs.size(1) <= dr);
+  TORCH_CHECK(positions.numel() == rows && row_seq.numel() == rows);
+  TORCH_CHECK(block_table.dim() == 2);
+  TORCH_CHECK(R <= 1024, "latent_attention: latent wider than 1024");
+  if (rows == 0) return;
+  const size_t lds = (size_t)(LAT_HB * (R + dr) + LAT_HB * LAT_CH) * 4;
+  TORCH_CHECK(lds <= 60 * 1024, "latent_attention: queries do not fit LDS");
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+  dim3 grid((unsigned)rows, (unsigned)((H + LAT_HB - 1) / LAT_HB));
+  KK_DISPATCH_ACT(q, {
+    if (R <= 256)
+      latent_attention_kernel<T, 1><<<grid, 256, lds, stream>>>(KK_ARGS);
+    else if (R <= 512)
+      latent_attention_kernel<T, 2><<<grid, 256, lds, stream>>>(KK_ARGS);
+    else
+      latent_attention_kernel<T, 4><<<grid, 256, lds, stream>>>(KK_ARGS);
+  });
+#undef KK_ARGS
+  HIP_CHECK_KERNEL();
+}
+
+}  // namespace kukeon

@@ -1,0 +1,170 @@
+// Selective state-space scan, the recurrent form:
+//   dt_t = softplus(dt_raw_t + dt_bias_h)
+//   S_t  = exp(-rate_h dt_t) S_(t-1) + dt_t B_t x_t^T        (S: N x P)
+//   y_t  = S_t^T C_t + skip_h x_t
+// One workgroup per (sequence, head). The state matrix stays in registers
+// for the whole portion: thread (p, l) owns rows n = l, l+LN, ... of column
+// p, so a step is NR fused multiply-adds per thread plus a reduction over
+// the LN neighbouring lanes. B, C, x and the step sizes of TT tokens are
+// staged in LDS at a time. All arithmetic is fp32; the state slot is read
+// once at the start of the portion (zeros at position 0, whatever the slot
+// held) and written once at its end. A single decoded token is a portion
+// of length one. Tokens are visited in order, so a position's result does
+// not depend on how the sequence was cut into portions.
+#include "elem.h"
+
+namespace kukeon {
+
+#define SSM_TT 16
+
+template <typename T, int NR>
+__global__ __launch_bounds__(1024) void ssm_scan_kernel(
+    float* __restrict__ y, const T* __restrict__ xbc, long ldx,
+    const T* __restrict__ dt, long lddt, const float* __restrict__ dt_bias,
+    const float* __restrict__ rate, const float* __restrict__ skip,
+    float* __restrict__ state, const int* __restrict__ positions,
+    const int* __restrict__ cu_rows, const int* __restrict__ state_slots,
+    int H, int P, int N, int G, int LN) {
+  extern __shared__ float sm[];
+  float* sB = sm;                       // [TT][N]
+  float* sC = sB + SSM_TT * N;          // [TT][N]
+  float* sX = sC + SSM_TT * N;          // [TT][P]
+  float* sDT = sX + SSM_TT * P;         // [TT]
+  float* sDE = sDT + SSM_TT;            // [TT]
+  const int s = blockIdx.x;
+  const int h = blockIdx.y;
+  const long row0 = cu_rows[s];
+  const int n = cu_rows[s + 1] - (int)row0;
+  if (n <= 0) return;
+  const int p0 = positions[row0];
+  if (p0 < 0) return;                   // inactive sequence
+  const int g = h / (H / G);
+  const int inner = H * P;
+  const int tid = threadIdx.x;
+  const int p = tid / LN;
+  const int l = tid - p * LN;
+  const bool live = p < P;
+  float* st = state + (((long)state_slots[s] * H + h) * N) * P;
+  float S[NR];
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const int nn = l + k * LN;
+    S[k] = (live && nn < N && p0 > 0) ? st[(long)nn * P + p] : 0.f;
+  }
+  const float bias_h = dt_bias[h];
+  const float rate_h = rate[h];
+  const float skip_h = skip[h];
+  for (int t0 = 0; t0 < n; t0 += SSM_TT) {
+    const int tt = min(SSM_TT, n - t0);
+    __syncthreads();
+    for (int i = tid; i < tt * N; i += blockDim.x) {
+      const int t = i / N, nn = i - t * N;
+      const T* row = xbc + (row0 + t0 + t) * ldx + inner + (long)g * N + nn;
+      sB[i] = ldf(row);
+      sC[i] = ldf(row + (long)G * N);
+    }
+    for (int i = tid; i < tt * P; i += blockDim.x) {
+      const int t = i / P, pp = i - t * P;
+      sX[i] = ldf(xbc + (row0 + t0 + t) * ldx + (long)h * P + pp);
+    }
+    for (int t = tid; t < tt; t += blockDim.x) {
+      const float v = ldf(dt + (row0 + t0 + t) * lddt + h) + bias_h;
+      const float sp = v > 20.f ? v : log1pf(expf(v));
+      sDT[t] = sp;
+      sDE[t] = expf(-rate_h * sp);
+    }
+    __syncthreads();
+    for (int t = 0; t < tt; ++t) {
+      const float x = live ? sX[t * P + p] : 0.f;
+      const float de = sDE[t];
+      const float dx = sDT[t] * x;
+      const float* bt = sB + t * N;
+      const float* ct = sC + t * N;
+      float acc = 0.f;
+#pragma unroll
+      for (int k = 0; k < NR; ++k) {
+        const int nn = l + k * LN;
+        if (nn < N) {
+          S[k] = fmaf(de, S[k], bt[nn] * dx);
+          acc = fmaf(S[k], ct[nn], acc);
+        }
+      }
+      for (int off = LN >> 1; off > 0; off >>= 1)
+        acc += __shfl_xor(acc, off, WAVE);
+      if (live && l == 0)
+        y[(row0 + t0 + t) * (long)inner + (long)h * P + p] =
+            fmaf(skip_h, x, acc);
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      const int nn = l + k * LN;
+      if (nn < N) st[(long)nn * P + p] = S[k];
+    }
+  }
+}
+
+// y [rows, H*P] fp32; xbc [rows, H*P + 2*G*N] = [x | B | C] (stride(1) ==
+// 1); dt [rows, H] (any row stride); dt_bias, rate, skip [H] fp32; state
+// [slots, H, N, P] fp32.
+void ssm_scan(torch::Tensor y, torch::Tensor xbc, torch::Tensor dt,
+              torch::Tensor dt_bias, torch::Tensor rate, torch::Tensor skip,
+              torch::Tensor state, torch::Tensor positions,
+              torch::Tensor cu_rows, torch::Tensor state_slots, int64_t H,
+              int64_t P, int64_t N, int64_t G) {
+  check_act(xbc, "xbc");
+  check_f32(y, "y"); check_f32(dt_bias, "dt_bias"); check_f32(rate, "rate");
+  check_f32(skip, "skip"); check_f32(state, "state");
+  check_i32(positions, "positions"); check_i32(cu_rows, "cu_rows");
+  check_i32(state_slots, "state_slots");
+  TORCH_CHECK(H >= 1 && P >= 1 && N >= 1 && G >= 1 && H % G == 0);
+  const long rows = xbc.size(0);
+  const long inner = H * P;
+  TORCH_CHECK(xbc.dim() == 2 && xbc.stride(1) == 1 &&
+              xbc.size(1) == inner + 2 * G * N);
+  TORCH_CHECK(dt.dim() == 2 && dt.size(0) == rows && dt.size(1) == H &&
+              dt.stride(1) == 1 && dt.scalar_type() == xbc.scalar_type());
+  TORCH_CHECK(y.dim() == 2 && y.size(0) == rows && y.size(1) == inner);
+  TORCH_CHECK(dt_bias.numel() == H && rate.numel() == H && skip.numel() == H);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == N &&
+              state.size(3) == P);
+  TORCH_CHECK(positions.numel() == rows);
+  const long nseq = cu_rows.numel() - 1;
+  TORCH_CHECK(nseq >= 1 && state_slots.numel() >= nseq);
+  if (rows == 0) return;
+  // lanes per state column: at most 16 rows of the state per thread, 32
+  // when the workgroup would otherwise exceed 1024 threads
+  int LN = 1;
+  while (LN * 16 < N && LN < 64) LN <<= 1;
+  int NR = 16;
+  if ((long)P * LN > 1024) {
+    LN = 1;
+    while (LN * 32 < N && LN < 64) LN <<= 1;
+    NR = 32;
+  }
+  TORCH_CHECK((long)LN * NR >= N && (long)P * LN <= 1024,
+              "ssm_scan: state ", N, " x ", P, " does not fit a workgroup");
+  const int threads = (int)((P * LN + 63) / 64 * 64);
+  const size_t lds = (size_t)SSM_TT * (2 * N + P + 2) * sizeof(float);
+  TORCH_CHECK(lds <= 64 * 1024, "ssm_scan: tile does not fit LDS");
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+  dim3 grid((unsigned)nseq, (unsigned)H);
+#define KK_ARGS y.data_ptr<float>(),                                        \
+        reinterpret_cast<const T*>(xbc.data_ptr()), (long)xbc.stride(0),    \
+        reinterpret_cast<const T*>(dt.data_ptr()), (long)dt.stride(0),      \
+        dt_bias.data_ptr<float>(), rate.data_ptr<float>(),                  \
+        skip.data_ptr<float>(), state.data_ptr<float>(),                    \
+        positions.data_ptr<int>(), cu_rows.data_ptr<int>(),                 \
+        state_slots.data_ptr<int>(), (int)H, (int)P, (int)N, (int)G, LN
+  KK_DISPATCH_ACT(xbc, {
+    if (NR == 16)
+      ssm_scan_kernel<T, 16><<<grid, threads, lds, stream>>>(KK_ARGS);
+    else
+      ssm_scan_kernel<T, 32><<<grid, threads, lds, stream>>>(KK_ARGS);
+  });
+#undef KK_ARGS
+  HIP_CHECK_KERNEL();
+}
+
+}  // namespace kukeon

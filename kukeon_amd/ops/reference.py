@@ -385,3 +385,187 @@ def diff_attention(out, q, k_cache, v_cache, gate, positions, row_seq,
             if gate is not None and gate.numel():
                 o = o * torch.sigmoid(gate[r, h].float())
             out[r, h * vdim:(h + 1) * vdim] = o.to(out.dtype)
+
+
+# ---------------------------------------------------------------------------
+# recurrent / latent group (state-space scan, short convolution with an
+# activation, latent attention, sandwich norms, table-routed experts)
+# ---------------------------------------------------------------------------
+
+def _unit_rms(x: torch.Tensor, eps: float) -> torch.Tensor:
+    return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def postnorm_residual_rmsnorm(x, y, post_w, w, eps: float, out) -> None:
+    """x (fp32, in place) += rmsnorm(y) * post_w; out = rmsnorm(x) * w."""
+    x += _unit_rms(y.float(), eps) * post_w
+    out.copy_((_unit_rms(x, eps) * w).to(out.dtype))
+
+
+def conv_act(out, proj, col0: int, cw, bias, state, positions, row_seq,
+             cu_rows, state_slots, act: int = 1) -> None:
+    """out = act(causal_conv(proj[:, col0:col0+C]) + bias) per sequence;
+    the taps before a portion come from the state slot (zeros before the
+    sequence start). cw [taps, C] with the newest tap last. act 1 = silu."""
+    taps, C = cw.shape
+    back = taps - 1
+    nseq = cu_rows.numel() - 1
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0 or int(positions[r0]) < 0:
+            continue
+        n = r1 - r0
+        p0 = int(positions[r0])
+        u = proj[r0:r1, col0: col0 + C].float()
+        hist = state[int(state_slots[s])].clone() if back else u[:0]
+        for k in range(back):
+            if p0 - back + k < 0:
+                hist[k] = 0
+        full = torch.cat([hist, u], 0)
+        y = torch.zeros(n, C)
+        for j in range(taps):
+            y = y + cw[j] * full[j: j + n]
+        y = y + bias
+        if act == 1:
+            y = y * torch.sigmoid(y)
+        out[r0:r1] = y.to(out.dtype)
+
+
+def ssm_scan(y, xbc, dt, dt_bias, rate, skip, state, positions, cu_rows,
+             state_slots, H: int, P: int, N: int, G: int) -> None:
+    """Selective scan, one token after the other. xbc [T, H*P + 2*G*N] =
+    [x | B | C]; dt [T, H] raw step sizes; state [slots, H, N, P] fp32;
+    y [T, H*P] fp32. Per head: S = exp(-rate softplus(dt + dt_bias)) S +
+    dt B x^T, y = S^T C + skip x."""
+    inner = H * P
+    nseq = cu_rows.numel() - 1
+    per = H // G
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0 or int(positions[r0]) < 0:
+            continue
+        slot = int(state_slots[s])
+        S = state[slot].clone()
+        if int(positions[r0]) == 0:
+            S.zero_()
+        for r in range(r0, r1):
+            x = xbc[r, :inner].float().view(H, P)
+            B = xbc[r, inner: inner + G * N].float().view(G, N)
+            C = xbc[r, inner + G * N:].float().view(G, N)
+            B = B.repeat_interleave(per, 0)                  # [H, N]
+            C = C.repeat_interleave(per, 0)
+            step = torch.nn.functional.softplus(
+                dt[r].float() + dt_bias, threshold=30.0)     # [H]
+            decay = torch.exp(-rate * step)
+            S = decay[:, None, None] * S + \
+                (step[:, None] * B)[:, :, None] * x[:, None, :]
+            y[r] = ((S * C[:, :, None]).sum(1) +
+                    skip[:, None] * x).reshape(inner)
+        state[slot] = S
+
+
+def gated_group_rmsnorm(out, y, z, w, groups: int, eps: float) -> None:
+    """out = rmsnorm_by_group(y * silu(z)) * w; the row is cut into
+    `groups` equal parts, each divided by its own root mean square."""
+    T, C = y.shape
+    zf = z.float()
+    g = y.float() * (zf * torch.sigmoid(zf))
+    g = _unit_rms(g.view(T, groups, C // groups), eps).view(T, C)
+    out.copy_((g * w).to(out.dtype))
+
+
+def _rot_pairs(v: torch.Tensor, ang: torch.Tensor, dims: int):
+    """v [..., n] one position; ang = [cos | sin] of dims/2 pairs."""
+    half = dims // 2
+    co, si = ang[:half], ang[half:]
+    out = v.clone()
+    a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+    out[..., 0:dims:2] = a * co - b * si
+    out[..., 1:dims:2] = b * co + a * si
+    return out
+
+
+def latent_kv_append(cq_out, cache, proj, q_col: int, kv_col: int, wq, wkv,
+                     eps: float, cs, positions, row_seq,
+                     block_table) -> None:
+    """cq_out = rmsnorm(proj[:, q_col:+Rq]) * wq; the cache row of every
+    token = [rmsnorm(proj[:, kv_col:+R]) * wkv | rotary(next dr columns)].
+    cache [blocks, 1, BS, R + dr]."""
+    Rq, R = wq.numel(), wkv.numel()
+    dr = cache.shape[3] - R
+    BS = cache.shape[2]
+    dims = cs.shape[1]
+    for r in range(proj.shape[0]):
+        p = int(positions[r])
+        if p < 0:
+            continue
+        row = proj[r].float()
+        cq_out[r] = (_unit_rms(row[q_col: q_col + Rq], eps) * wq).to(
+            cq_out.dtype)
+        c = _unit_rms(row[kv_col: kv_col + R], eps) * wkv
+        kr = _rot_pairs(row[kv_col + R: kv_col + R + dr], cs[p], dims)
+        blk = int(block_table[int(row_seq[r]), p // BS])
+        cache[blk, 0, p % BS] = torch.cat([c, kr]).to(cache.dtype)
+
+
+def latent_attention(out, q_abs, q, cache, cs, positions, row_seq,
+                     block_table, H: int, dn: int, dr: int, window: int,
+                     scale: float) -> None:
+    """Attention of H heads over ONE shared cache row per token,
+    [latent (R) | rotated key part (dr)]. q_abs [H, T, R] is the query
+    already multiplied into latent space; q [T, H*(dn+dr)] holds the
+    unrotated rotary part of every head behind its first dn entries.
+    out [H, T, R] = softmax-weighted sum of the latents over the last
+    `window` positions."""
+    R = q_abs.shape[2]
+    BS = cache.shape[2]
+    dims = cs.shape[1]
+    T = q.shape[0]
+    for r in range(T):
+        p = int(positions[r])
+        if p < 0:
+            out[:, r] = 0
+            continue
+        s = int(row_seq[r])
+        lo = max(0, p - window + 1) if window > 0 else 0
+        js = torch.arange(lo, p + 1)
+        blk = block_table[s, (js // BS).long()].long()
+        rows = cache[blk, 0, (js % BS).long()].float()       # [n, R+dr]
+        qr = _rot_pairs(q[r, : H * (dn + dr)].float().view(H, dn + dr)[:, dn:], cs[p], dims)
+        sc = (q_abs[:, r].float() @ rows[:, :R].T +
+              qr @ rows[:, R:].T) * scale                    # [H, n]
+        w = torch.softmax(sc, -1)
+        out[:, r] = (w @ rows[:, :R]).to(out.dtype)
+
+
+def head_gate(out, o, gate) -> None:
+    """out[t, h*dv:(h+1)*dv] = o[h, t] * sigmoid(gate[t, h])."""
+    Hh, T, dv = o.shape
+    g = torch.sigmoid(gate.float())                          # [T, H]
+    out.copy_((o.float().permute(1, 0, 2) * g[:, :, None]).reshape(
+        T, Hh * dv).to(out.dtype))
+
+
+def xielu(out, z, ap: float, aq: float) -> None:
+    """z > 0: ap z^2 + z/2;  z <= 0: aq (exp(z) - 1 - z) + z/2."""
+    zf = z.float()
+    pos = ap * zf * zf + 0.5 * zf
+    neg = aq * (torch.expm1(zf.clamp(max=0.0)) - zf) + 0.5 * zf
+    out.copy_(torch.where(zf > 0, pos, neg).to(out.dtype))
+
+
+def table_moe(out, h, ids, table, w_up, w_down) -> None:
+    """out[t] = mean over the experts table[ids[t]] of
+    w_down[e] relu(w_up[e] h[t])^2."""
+    top = table.shape[1]
+    for r in range(h.shape[0]):
+        acc = torch.zeros(h.shape[1])
+        for e in table[int(ids[r])].tolist():
+            a = torch.relu(torch.nn.functional.linear(h[r], w_up[e]))
+            a = (a.float() ** 2).to(h.dtype)
+            acc += torch.nn.functional.linear(a, w_down[e]).float()
+        out[r] = (acc / top).to(out.dtype)
+
+
+def softcap_(logits, cap: float) -> None:
+    logits.copy_(cap * torch.tanh(logits / cap))

@@ -54,7 +54,7 @@ def main(argv=None) -> int:
 
     with open(os.path.join(args.model, "config.json")) as f:
         arch = json.load(f).get("architecture")
-    from kukeon_amd.models.registry import ARCHITECTURES
+    from kukeon_amd.models.registry import ARCHITECTURES, OP_GROUPS
     if arch not in ARCHITECTURES:
         print(f"no model class for architecture {arch!r}", file=sys.stderr)
         return 2
@@ -62,7 +62,7 @@ def main(argv=None) -> int:
     import torch
     device = args.device or ("cuda:0" if torch.cuda.is_available() else "cpu")
     if device.startswith("cuda"):
-        _ensure_built(("mix",))
+        _ensure_built(OP_GROUPS[ARCHITECTURES[arch]])
     # exact mode: no reduced-precision matrix products
     torch.backends.cuda.matmul.allow_tf32 = False
     torch.set_float32_matmul_precision("highest")

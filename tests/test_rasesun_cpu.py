@@ -1,0 +1,109 @@
+"""Rasesun family on the CPU path (fp32 reference ops through the engine)
+against the plain model in rasesun_oracle.py."""
+import os
+import sys
+
+import pytest
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+import rasesun_cases as cases  # noqa: E402
+
+DEV, DT = "cpu", "fp32"
+
+
+@pytest.mark.parametrize("name", sorted(cases.CONFIGS))
+def test_whole_prompt(name):
+    cases.case_whole(name, DEV, DT)
+
+
+def test_residual_after_every_layer_run():
+    cases.case_layers(DEV, DT)
+
+
+@pytest.mark.parametrize("name", ["hybrid", "looped"])
+def test_prefill_against_token_by_token(name):
+    cases.case_prefill_vs_decode(name, DEV, DT)
+
+
+@pytest.mark.parametrize("sizes", [(2,), (3, 2, 7), (16, 1, 5)])
+def test_portions(sizes):
+    cases.case_portions("hybrid", DEV, DT, sizes)
+
+
+def test_unequal_batch():
+    cases.case_batch("hybrid", DEV, DT)
+
+
+def test_pages_and_slots_reused():
+    cases.case_reuse(DEV, DT)
+
+
+def test_first_tokens():
+    cases.case_first_tokens(DEV, DT)
+
+
+def test_long_decode():
+    cases.case_long_decode(DEV, DT)
+
+
+def test_greedy_generation():
+    cases.case_greedy(DEV, DT)
+
+
+def test_checkpoint_folder(tmp_path):
+    cases.case_registry(tmp_path, DEV, DT)
+
+
+def test_op_sandwich_norm():
+    cases.case_op_sandwich_norm(DEV, DT)
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4])
+def test_op_conv(taps):
+    cases.case_op_conv(DEV, DT, taps=taps)
+
+
+def test_op_scan():
+    cases.case_op_scan(DEV, DT)
+    cases.case_op_scan(DEV, DT, H=4, P=3, N=40, G=1, cuts=(1, 1, 20, 2))
+
+
+def test_op_gated_norm():
+    cases.case_op_gated_norm(DEV, DT)
+
+
+def test_op_activations():
+    cases.case_op_activations(DEV, DT)
+
+
+@pytest.mark.parametrize("top", [1, 2, 3])
+def test_op_table_moe(top):
+    cases.case_op_table_moe(DEV, DT, top=top)
+
+
+def test_op_latent_append():
+    cases.case_op_latent_append(DEV, DT)
+
+
+def test_op_latent_attention():
+    cases.case_op_latent_attention(DEV, DT, ctx=120, window=40)
+
+
+def test_config_rejects_unknown_parts():
+    from kukeon_amd.models.rasesun import RasesunConfig
+    cfg = cases.CONFIGS["hybrid"]()
+    cfg["layers"][0]["type"] = "other"
+    with pytest.raises(ValueError):
+        RasesunConfig.from_json(cfg)
+    cfg = cases.CONFIGS["hybrid"]()
+    cfg["layers"][0]["mlp"]["kind"] = "other"
+    with pytest.raises(ValueError):
+        RasesunConfig.from_json(cfg)
+
+
+def test_layer_runs_follow_the_loop():
+    from kukeon_amd.models.rasesun import RasesunConfig
+    c = RasesunConfig.from_json(cases.CONFIGS["hybrid"]())
+    assert c.runs() == [0, 1, 2, 1, 2, 1, 2, 3]
+    c = RasesunConfig.from_json(cases.CONFIGS["wide"]())
+    assert c.runs() == [0, 1]
