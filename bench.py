@@ -30,16 +30,20 @@ COMPARE_SIZES = {
 
 
 def compare_families(args) -> None:
-    """Prefill and decode tokens/s of Lipedra and Llama through the same
-    engine at equal sizes: same width, head counts, feed-forward size,
-    layer count, vocabulary and cache bytes per token (Llama head_dim 128;
-    Lipedra two score maps of 64 and value rows of 128)."""
+    """Prefill and decode tokens/s of Lipedra or Rasesun and of Llama
+    through the same engine at equal sizes: same width, head counts,
+    feed-forward size, layer count and vocabulary (Llama head_dim 128;
+    Lipedra two score maps of 64 and value rows of 128 — equal cache bytes
+    per token; Rasesun three state-space layers to one latent-attention
+    layer with a 1024-token window, every second feed-forward a mixture of
+    16 table-routed experts, two active)."""
     from kukeon_amd.engine.config import (EngineConfig, ModelConfig,
                                           SamplingParams)
     from kukeon_amd.engine.engine import LLMEngine
     from kukeon_amd.engine.kv_cache import SequenceKV
     from kukeon_amd.models import registry
     from kukeon_amd.models.lipedra import lipedra_bench
+    from kukeon_amd.models.rasesun import rasesun_bench
 
     device = args.device or ("cuda:0" if torch.cuda.is_available() else "cpu")
     on_gpu = device != "cpu"
@@ -50,13 +54,19 @@ def compare_families(args) -> None:
         W, hq, hk, ff, nl = COMPARE_SIZES[size]
         if not on_gpu:
             W, hq, hk, ff, nl = 256, 2, 2, 512, 2
-        for fam in ("llama", "lipedra"):
+        for fam in ("llama", args.compare_family):
             if fam == "llama":
                 cfg = ModelConfig(name=f"llama-{size}", hidden_size=W,
                                   num_layers=nl, num_q_heads=hq,
                                   num_kv_heads=hk, head_dim=128,
                                   intermediate_size=ff, vocab_size=vocab,
                                   max_position=4096)
+            elif fam == "rasesun":
+                cfg = rasesun_bench(width=W, layers=nl, heads=hq, ff=ff,
+                                    vocab=vocab, attn_every=min(4, nl),
+                                    window=1024 if on_gpu else 16,
+                                    experts=16 if on_gpu else 4,
+                                    name=f"rasesun-{size}")
             else:
                 cfg = lipedra_bench(width=W, layers=nl, heads=hq,
                                     kv_heads=hk, dim=64, vdim=128, ff=ff,
@@ -139,6 +149,10 @@ def main() -> None:
                     help="instead of the headline workload: prefill and "
                          "decode throughput of the Lipedra family beside "
                          "Llama at equal layer sizes (random weights)")
+    ap.add_argument("--compare-family", default="lipedra",
+                    choices=["lipedra", "rasesun"],
+                    help="with --compare-families: the family that runs "
+                         "beside Llama")
     ap.add_argument("--compare-sizes", default="2k,4k,8k",
                     help="with --compare-families: which of 2k,4k,8k")
     args = ap.parse_args()

@@ -421,6 +421,7 @@ class LLMEngine:
             meta.state = self.states.layers if self.states else None
             meta.max_rows = max(len(t) for _, t in items)
             meta.chunk_lens = [len(t) for _, t in items]
+            meta.host_ids = ids
         return self.model.forward(i32(ids), self.kv.k, self.kv.v, meta)
 
     def forward_tokens(self, entries, want=None) -> torch.Tensor:

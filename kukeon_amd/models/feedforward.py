@@ -46,7 +46,8 @@ class XieluFF(nn.Module):
     def tensor_shapes(f: FFCfg, width: int, vocab: int) -> Dict[str, tuple]:
         return {"up": (f.ff, width), "down": (width, f.ff), "act": (2,)}
 
-    def forward(self, h: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, ids: torch.Tensor,
+                meta=None) -> torch.Tensor:
         z = ops.linear(h, self.w_up)
         a = torch.empty_like(z)
         ops.xielu(a, z, self.ap, self.aq)
@@ -75,6 +76,7 @@ class TableMoE(nn.Module):
         if int(table.min()) < 0 or int(table.max()) >= f.experts:
             raise ValueError(f"{p}table names an expert that does not exist")
         self.table = table.to(device).contiguous()
+        self.table_host = table.cpu().numpy()
 
     @staticmethod
     def tensor_shapes(f: FFCfg, width: int, vocab: int) -> Dict[str, tuple]:
@@ -84,7 +86,52 @@ class TableMoE(nn.Module):
             out[f"e{e}.down"] = (width, f.ff)
         return out
 
-    def forward(self, h: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    # portions of at least this many rows take the grouped form when the
+    # step's token ids are known on the host
+    grouped_min_rows = 64
+
+    def forward(self, h: torch.Tensor, ids: torch.Tensor,
+                meta=None) -> torch.Tensor:
         out = torch.empty_like(h)
+        host_ids = getattr(meta, "host_ids", None)
+        if host_ids is not None and h.shape[0] >= self.grouped_min_rows:
+            return self._forward_grouped(out, h, host_ids, meta)
         ops.table_moe(out, h, ids, self.table, self.w_up, self.w_down)
+        return out
+
+    def _forward_grouped(self, out, h, host_ids, meta) -> torch.Tensor:
+        """Rows sorted by expert on the host (the routing is a function of
+        the token id, which the scheduler knows): no device round trip to
+        learn the group sizes, and every expert runs plain GEMMs over its
+        contiguous rows."""
+        import numpy as np
+        T, W = h.shape
+        top, E = self.f.top, self.f.experts
+        key = ("table_moe", id(self))
+        maps = meta.tile_maps.get(key)
+        if maps is None:
+            flat = self.table_host[np.asarray(host_ids)].reshape(-1)
+            order = np.argsort(flat, kind="stable")
+            counts = np.bincount(flat, minlength=E)
+            inv = np.empty_like(order)
+            inv[order] = np.arange(order.size)
+            dev = h.device
+            maps = (torch.from_numpy((order // top).astype(np.int32)).to(dev),
+                    torch.from_numpy(inv.astype(np.int32).reshape(T, top))
+                    .to(dev), counts.tolist())
+            meta.tile_maps[key] = maps
+        row_map, inv, counts = maps
+        rows = torch.empty(T * top, W, dtype=h.dtype, device=h.device)
+        ops.gather_rows(rows, h, row_map)
+        done = torch.empty_like(rows)
+        at = 0
+        for e in range(E):
+            n = counts[e]
+            if n == 0:
+                continue
+            a = ops.linear(rows[at: at + n], self.w_up[e])
+            ops.relu_square_(a)
+            done[at: at + n] = ops.linear(a, self.w_down[e])
+            at += n
+        ops.combine_rows(out, done, inv)
         return out

@@ -45,6 +45,9 @@ class AttnMeta:
     max_rows: int = 0                         # longest portion in the batch
     chunk_lens: Optional[list] = None         # host: rows per sequence
     tile_maps: dict = field(default_factory=dict)  # per-step kernel maps
+    # the step's token ids as the scheduler holds them (None when they
+    # exist on the device only, as inside a captured decode graph)
+    host_ids: Optional[list] = None
 
 
 def split_prefill_meta(meta: AttnMeta, parts: int = 2):

@@ -129,6 +129,38 @@ class RasesunConfig:
             layers=layers)
 
 
+def rasesun_bench(width=4096, layers=8, heads=32, ff=14336, vocab=128256,
+                  attn_every=4, window=1024, experts=16, top=2,
+                  name="rasesun-8b-like") -> RasesunConfig:
+    """A layer stack at real-model sizes (random weights) for throughput
+    runs: every `attn_every`-th layer is latent attention (heads of 128
+    unrotated + 64 rotated entries, a 512-wide latent), the others are
+    state-space layers of twice the width (64-channel heads, 128 state
+    rows, 8 groups); feed-forwards alternate between dense and
+    table-routed experts of the same total active size."""
+    ls = []
+    for i in range(layers):
+        if i % attn_every == attn_every - 1:
+            kind = "latent_attention"
+            mix = LatentAttnCfg(heads=heads, dim=128, rot_dim=64, vdim=128,
+                                q_rank=max(64, width * 3 // 8), kv_rank=512,
+                                scale=192 ** -0.5, window=window,
+                                rot_dims=64, rot_base=10000.0)
+        else:
+            kind = "mamba2"
+            mix = StateSpaceCfg(heads=2 * width // 64, vdim=64, state=128,
+                                groups=8, conv=4, norm_groups=8)
+        if i % 2:
+            mlp = FFCfg("moe", max(8, ff // top // 8 * 8), experts=experts,
+                        top=top)
+        else:
+            mlp = FFCfg("dense", ff)
+        ls.append(RasesunLayerCfg(kind, mix, mlp))
+    return RasesunConfig(name=name, width=width, vocab_size=vocab,
+                         embed_scale=1.0, rms_eps=1e-6, logit_softcap=30.0,
+                         layers=ls)
+
+
 def tensor_shapes(cfg: RasesunConfig) -> Dict[str, tuple]:
     """Names and shapes of a checkpoint of this configuration."""
     W = cfg.width
@@ -295,7 +327,7 @@ class RasesunModel(nn.Module):
             if layer.ff is not None:
                 ops.postnorm_residual_rmsnorm(x, y, layer.norm1b,
                                               layer.norm2, eps, h)
-                y = layer.ff(h, input_ids)
+                y = layer.ff(h, input_ids, meta)
                 h = torch.empty_like(h)
                 ops.postnorm_residual_rmsnorm(x, y, layer.norm2b, nxt, eps, h)
             else:

@@ -89,13 +89,35 @@ LIPEDRA_PRESETS = {
 }
 
 
+def _rasesun_preset(**kw):
+    def make():
+        from kukeon_amd.models.rasesun import rasesun_bench
+        return rasesun_bench(**kw)
+    return make
+
+
+# random-weight Rasesun stacks: three state-space layers to one latent
+# attention layer at Llama-3-8B width, and a small one for tests
+RASESUN_PRESETS = {
+    "rasesun-8b-like": _rasesun_preset(width=4096, layers=32, heads=32,
+                                       ff=14336, vocab=128256,
+                                       name="rasesun-8b-like"),
+    "tiny-rasesun": _rasesun_preset(width=128, layers=4, heads=2, ff=256,
+                                    vocab=384, window=24, experts=4,
+                                    name="tiny-rasesun"),
+}
+
+
 def preset_names():
-    return sorted(list(MODEL_PRESETS) + list(LIPEDRA_PRESETS))
+    return sorted(list(MODEL_PRESETS) + list(LIPEDRA_PRESETS) +
+                  list(RASESUN_PRESETS))
 
 
 def preset(name: str):
     if name in LIPEDRA_PRESETS:
         return LIPEDRA_PRESETS[name]()
+    if name in RASESUN_PRESETS:
+        return RASESUN_PRESETS[name]()
     if name not in MODEL_PRESETS:
         raise KeyError(f"unknown model preset {name!r}; known: "
                        f"{preset_names()}")

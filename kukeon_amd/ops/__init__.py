@@ -531,5 +531,17 @@ def table_moe(out, h, ids, table, w_up, w_down) -> None:
     _recur(h).table_moe(out, h, ids, table, w_up, w_down)
 
 
+def gather_rows(out, inp, row_map) -> None:
+    _recur(out).gather_rows(out, inp, row_map)
+
+
+def relu_square_(x) -> None:
+    _recur(x).relu_square_(x)
+
+
+def combine_rows(out, inp, inv) -> None:
+    _recur(out).combine_rows(out, inp, inv)
+
+
 def softcap_(logits, cap: float) -> None:
     _recur(logits).softcap_(logits, cap)

@@ -44,6 +44,9 @@ void latent_attention(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q,
                       int64_t dr, int64_t window, double scale);
 void table_moe(torch::Tensor out, torch::Tensor h, torch::Tensor ids,
                torch::Tensor table, torch::Tensor w_up, torch::Tensor w_down);
+void gather_rows(torch::Tensor out, torch::Tensor in, torch::Tensor map);
+void relu_square_(torch::Tensor x);
+void combine_rows(torch::Tensor out, torch::Tensor in, torch::Tensor inv);
 }  // namespace kukeon
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -67,6 +70,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "norm the latents, rotate the shared key part, write the cache row");
   m.def("latent_attention", &kukeon::latent_attention,
         "windowed attention over the shared latent cache row");
+  m.def("gather_rows", &kukeon::gather_rows, "out[r] = in[map[r]]");
+  m.def("relu_square_", &kukeon::relu_square_, "x <- relu(x)^2, in place");
+  m.def("combine_rows", &kukeon::combine_rows,
+        "out[t] = mean over k of in[inv[t, k]]");
   m.def("table_moe", &kukeon::table_moe,
         "experts chosen by a token-id table, relu^2, equal weights");
 }

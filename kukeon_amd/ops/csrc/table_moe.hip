@@ -126,4 +126,96 @@ void table_moe(torch::Tensor out, torch::Tensor h, torch::Tensor ids,
   HIP_CHECK_KERNEL();
 }
 
+// ---- grouped form for long portions ---------------------------------------
+// With the token ids known on the host, the (token, expert) pairs are sorted
+// by expert there; the device gathers the rows in that order, every expert
+// runs two vendor GEMMs over its contiguous rows with relu^2 in between, and
+// combine_rows folds each token's `top` results with equal weights.
+
+template <typename T>
+__global__ __launch_bounds__(256) void gather_rows_kernel(
+    T* __restrict__ out, const T* __restrict__ in, const int* __restrict__ map,
+    int W) {
+  const long r = blockIdx.x;
+  const T* src = in + (long)map[r] * W;
+  T* dst = out + r * (long)W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) dst[i] = src[i];
+}
+
+// out [n, W] = in[map[r], :]
+void gather_rows(torch::Tensor out, torch::Tensor in, torch::Tensor map) {
+  check_act(out, "out"); check_act(in, "in"); check_i32(map, "map");
+  TORCH_CHECK(out.dim() == 2 && in.dim() == 2 && out.is_contiguous() &&
+              in.is_contiguous() && out.size(1) == in.size(1) &&
+              out.scalar_type() == in.scalar_type() &&
+              map.numel() == out.size(0));
+  const long n = out.size(0);
+  if (n == 0) return;
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+  KK_DISPATCH_ACT(out, {
+    gather_rows_kernel<T><<<dim3((unsigned)n), 256, 0, stream>>>(
+        reinterpret_cast<T*>(out.data_ptr()),
+        reinterpret_cast<const T*>(in.data_ptr()), map.data_ptr<int>(),
+        (int)out.size(1));
+  });
+  HIP_CHECK_KERNEL();
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void relu_square_kernel(T* __restrict__ x,
+                                                          long total) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const float v = fmaxf(ldf(x + i), 0.f);
+  stf(x + i, v * v);
+}
+
+void relu_square_(torch::Tensor x) {
+  check_act(x, "x");
+  TORCH_CHECK(x.is_contiguous());
+  const long total = x.numel();
+  if (total == 0) return;
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+  KK_DISPATCH_ACT(x, {
+    relu_square_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0,
+                            stream>>>(reinterpret_cast<T*>(x.data_ptr()),
+                                      total);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void combine_rows_kernel(
+    T* __restrict__ out, const T* __restrict__ in, const int* __restrict__ inv,
+    int W, int top) {
+  const long t = blockIdx.x;
+  const float share = 1.0f / (float)top;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k)
+      acc += ldf(in + (long)inv[t * top + k] * W + i);
+    stf(out + t * (long)W + i, acc * share);
+  }
+}
+
+// out [T, W] = mean_k in[inv[t, k], :]
+void combine_rows(torch::Tensor out, torch::Tensor in, torch::Tensor inv) {
+  check_act(out, "out"); check_act(in, "in"); check_i32(inv, "inv");
+  TORCH_CHECK(out.dim() == 2 && in.dim() == 2 && out.is_contiguous() &&
+              in.is_contiguous() && out.size(1) == in.size(1) &&
+              out.scalar_type() == in.scalar_type());
+  TORCH_CHECK(inv.dim() == 2 && inv.size(0) == out.size(0) &&
+              inv.size(0) * inv.size(1) == in.size(0));
+  const long n = out.size(0);
+  if (n == 0) return;
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+  KK_DISPATCH_ACT(out, {
+    combine_rows_kernel<T><<<dim3((unsigned)n), 256, 0, stream>>>(
+        reinterpret_cast<T*>(out.data_ptr()),
+        reinterpret_cast<const T*>(in.data_ptr()), inv.data_ptr<int>(),
+        (int)out.size(1), (int)inv.size(1));
+  });
+  HIP_CHECK_KERNEL();
+}
+
 }  // namespace kukeon

@@ -569,3 +569,16 @@ def table_moe(out, h, ids, table, w_up, w_down) -> None:
 
 def softcap_(logits, cap: float) -> None:
     logits.copy_(cap * torch.tanh(logits / cap))
+
+
+def gather_rows(out, inp, row_map) -> None:
+    out.copy_(inp[row_map.long()])
+
+
+def relu_square_(x) -> None:
+    x.copy_((torch.relu(x.float()) ** 2).to(x.dtype))
+
+
+def combine_rows(out, inp, inv) -> None:
+    """out[t] = mean over k of inp[inv[t, k]]."""
+    out.copy_(inp[inv.long()].float().mean(1).to(out.dtype))

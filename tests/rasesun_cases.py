@@ -375,6 +375,26 @@ def case_window_chunks(device, dtype):
     check(got, want, dtype, "portions and decoding")
 
 
+def case_grouped_experts(device, dtype):
+    """Long portions sort their rows by expert and run each expert over its
+    rows at once; short ones go token by token. Both against the plain
+    model, two experts per token, two requests in the long step."""
+    cfg = CONFIGS["hybrid"]()
+    W = weights(cfg, 12)
+    prompts = [tokens(cfg, n, 70 + n) for n in (90, 71)]
+    want = [oracle.forward(cfg, W, p) for p in prompts]
+    eng = make_engine(cfg, W, device, dtype, blocks=64, max_len=128)
+    got = run_schedule(eng, prompts, [[(0, 90), (1, 70)], [(1, 1)]])
+    for i in range(2):
+        check(got[i], want[i], dtype, f"sorted rows, request {i}")
+    a, b = portions(90, (7,)), portions(71, (5, 1))
+    sched = [[(i, c[k]) for i, c in ((0, a), (1, b)) if k < len(c)]
+             for k in range(max(len(a), len(b)))]
+    got = run_schedule(eng, prompts, sched)
+    for i in range(2):
+        check(got[i], want[i], dtype, f"token by token, request {i}")
+
+
 def case_greedy(device, dtype, graphs=False):
     """Generation through add_request / step with the greedy sampler."""
     cfg = CONFIGS["hybrid"]()

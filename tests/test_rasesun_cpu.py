@@ -46,6 +46,10 @@ def test_long_decode():
     cases.case_long_decode(DEV, DT)
 
 
+def test_long_portions_sort_rows_by_expert():
+    cases.case_grouped_experts(DEV, DT)
+
+
 def test_greedy_generation():
     cases.case_greedy(DEV, DT)
 

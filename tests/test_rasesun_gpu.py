@@ -120,6 +120,11 @@ def test_window_longer_than_a_key_chunk(dtype):
 
 
 @BOTH
+def test_long_portions_sort_rows_by_expert(dtype):
+    cases.case_grouped_experts(DEV, dtype)
+
+
+@BOTH
 @pytest.mark.parametrize("graphs", [False, True])
 def test_greedy_generation(dtype, graphs):
     cases.case_greedy(DEV, dtype, graphs=graphs)
