@@ -78,6 +78,222 @@ __global__ __launch_bounds__(256) void table_moe_down_kernel(
   }
 }
 
+// ---- expert-major form for small batches ---------------------------------
+// A decode step brings a few dozen tokens that share a handful of experts.
+// Here a workgroup belongs to (expert, tile of output rows): it lists the
+// (token, k) pairs routed to its expert, and each wave keeps one weight row
+// in registers while it walks that list, so an expert's weights leave HBM
+// once per step however many tokens use it. A pair's dot product is summed
+// in an order fixed by the row length alone, never by the batch.
+#define MOE_MAX_PAIRS 2048
+#define MOE_SEG 16              // 8-element chunks of a row held per lane
+
+DEV_INLINE int moe_list_pairs(int* list, int* count,
+                              const int* __restrict__ ids,
+                              const int* __restrict__ table, int pairs,
+                              int top, int vocab, int e) {
+  if (threadIdx.x == 0) *count = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    int id = ids[i / top];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    if (table[(long)id * top + i % top] == e) list[atomicAdd(count, 1)] = i;
+  }
+  __syncthreads();
+  return *count;
+}
+
+// one weight row (K elements, K % 8 == 0) against the rows src[pair * lds]
+// of all listed pairs; FN(pair, value) consumes each result on lane 0
+template <typename T, typename F>
+DEV_INLINE void moe_row_times_pairs(const T* __restrict__ wrow, int K,
+                                    const T* __restrict__ src, long lds,
+                                    int div, const int* list, int n, F fn) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int chunks = K / 8;
+  for (int seg0 = 0; seg0 < chunks; seg0 += MOE_SEG * WAVE) {
+    Raw8<T> w[MOE_SEG];
+#pragma unroll
+    for (int c = 0; c < MOE_SEG; ++c) {
+      const int ch = seg0 + c * WAVE + lane;
+      if (ch < chunks) w[c].load(wrow + (long)ch * 8);
+    }
+    for (int j = 0; j < n; ++j) {
+      const int pair = list[j];
+      const T* x = src + (long)(pair / div) * lds;
+      float acc = 0.f;
+#pragma unroll
+      for (int c = 0; c < MOE_SEG; ++c) {
+        const int ch = seg0 + c * WAVE + lane;
+        if (ch < chunks) {
+          Raw8<T> xv;
+          xv.load(x + (long)ch * 8);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc = fmaf(w[c].get(k), xv.get(k), acc);
+        }
+      }
+      acc = wave_sum(acc);
+      fn(pair, acc, seg0 == 0);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void table_moe_up_expert_kernel(
+    T* __restrict__ act, float* __restrict__ part, const T* __restrict__ h,
+    const int* __restrict__ ids, const int* __restrict__ table,
+    const T* __restrict__ w_up, int W, int ff, int top, int vocab,
+    int pairs) {
+  __shared__ int list[MOE_MAX_PAIRS];
+  __shared__ int count;
+  const int e = blockIdx.x;
+  const int n = moe_list_pairs(list, &count, ids, table, pairs, top, vocab, e);
+  if (n == 0) return;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wave = threadIdx.x / WAVE;
+  const int f0 = (blockIdx.y * 4 + wave) * MOE_ROWS_PER_WAVE;
+  const bool one_seg = W / 8 <= MOE_SEG * WAVE;
+  for (int j = 0; j < MOE_ROWS_PER_WAVE; ++j) {
+    const int f = f0 + j;
+    if (f >= ff) break;
+    const T* wr = w_up + ((long)e * ff + f) * W;
+    moe_row_times_pairs<T>(
+        wr, W, h, (long)W, top, list, n,
+        [&](int pair, float v, bool first) {
+          if (lane != 0) return;
+          if (one_seg) {
+            const float r = fmaxf(v, 0.f);
+            stf(act + (long)pair * ff + f, r * r);
+          } else {       // long rows: sum the segments in fp32 first
+            float* p = part + (long)pair * ff + f;
+            *p = first ? v : *p + v;
+          }
+        });
+    if (!one_seg && lane == 0) {
+      for (int jj = 0; jj < n; ++jj) {
+        const long at = (long)list[jj] * ff + f;
+        const float r = fmaxf(part[at], 0.f);
+        stf(act + at, r * r);
+      }
+    }
+  }
+}
+
+// part[pair, c] = W_down[e][c, :] . act[pair, :]
+template <typename T>
+__global__ __launch_bounds__(256) void table_moe_down_expert_kernel(
+    float* __restrict__ part, const T* __restrict__ act,
+    const int* __restrict__ ids, const int* __restrict__ table,
+    const T* __restrict__ w_down, int W, int ff, int top, int vocab,
+    int pairs) {
+  __shared__ int list[MOE_MAX_PAIRS];
+  __shared__ int count;
+  const int e = blockIdx.x;
+  const int n = moe_list_pairs(list, &count, ids, table, pairs, top, vocab, e);
+  if (n == 0) return;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wave = threadIdx.x / WAVE;
+  const int c0 = (blockIdx.y * 4 + wave) * MOE_ROWS_PER_WAVE;
+  for (int j = 0; j < MOE_ROWS_PER_WAVE; ++j) {
+    const int c = c0 + j;
+    if (c >= W) break;
+    const T* wr = w_down + ((long)e * W + c) * ff;
+    moe_row_times_pairs<T>(wr, ff, act, (long)ff, 1, list, n,
+                           [&](int pair, float v, bool first) {
+                             if (lane != 0) return;
+                             float* p = part + (long)pair * W + c;
+                             *p = first ? v : *p + v;
+                           });
+  }
+}
+
+// out[t, :] = (1/top) sum_k part[t*top + k, :], k in order
+template <typename T>
+__global__ __launch_bounds__(256) void table_moe_mean_kernel(
+    T* __restrict__ out, const float* __restrict__ part, long total, int W,
+    int top) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long t = i / W;
+  const int c = (int)(i - t * W);
+  float acc = 0.f;
+  for (int k = 0; k < top; ++k) acc += part[(t * top + k) * W + c];
+  stf(out + i, acc * (1.0f / (float)top));
+}
+
+// ---- expert-major form on the matrix cores (bf16) -------------------------
+// The same split of work, with v_mfma_f32_16x16x32_bf16: a wave owns 16
+// weight rows (the A operand, lane = row, 8 consecutive k per lane) and up
+// to 16 listed pairs at a time (the B operand, lane = pair). Each lane
+// fetches 64 contiguous bytes of its weight row and of its pair's input per
+// 128-wide k block; the same k permutation on both operands leaves the
+// product unchanged. Output lane (pair = l & 15) holds rows 4 * (l >> 4) + r.
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short moe_bf16x8_v;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float moe_f32x4_v;
+DEV_INLINE moe_bf16x8_v moe_frag(const uint4& v) {
+  return __builtin_bit_cast(moe_bf16x8_v, v);
+}
+
+// UP:   dst = act  [pairs, NR] bf16, relu(.)^2, source rows h[pair / top]
+// !UP:  dst = part [pairs, NR] fp32, source rows act[pair]
+template <bool UP>
+__global__ __launch_bounds__(256) void table_moe_mfma_kernel(
+    void* __restrict__ dst, const bf16_t* __restrict__ src,
+    const int* __restrict__ ids, const int* __restrict__ table,
+    const bf16_t* __restrict__ w, int NR, int K, int top, int vocab,
+    int pairs) {
+  __shared__ int list[MOE_MAX_PAIRS];
+  __shared__ int count;
+  const int e = blockIdx.x;
+  const int n = moe_list_pairs(list, &count, ids, table, pairs, top, vocab, e);
+  if (n == 0) return;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wave = threadIdx.x / WAVE;
+  const int rc = lane & 15;
+  const int g4 = lane >> 4;
+  const int r0 = (blockIdx.y * 4 + wave) * 16;
+  if (r0 >= NR) return;
+  const int arow = min(r0 + rc, NR - 1);
+  const bf16_t* wrow = w + ((long)e * NR + arow) * K + g4 * 32;
+  for (int g0 = 0; g0 < n; g0 += 16) {
+    const int pair = g0 + rc < n ? list[g0 + rc] : -1;
+    const bf16_t* xrow =
+        src + (long)(pair < 0 ? 0 : (UP ? pair / top : pair)) * K + g4 * 32;
+    moe_f32x4_v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+    for (int k0 = 0; k0 < K; k0 += 128) {
+      uint4 a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        a[i] = *reinterpret_cast<const uint4*>(wrow + k0 + i * 8);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        b[i] = pair < 0 ? uint4{0u, 0u, 0u, 0u}
+                        : *reinterpret_cast<const uint4*>(xrow + k0 + i * 8);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_frag(a[i]),
+                                                      moe_frag(b[i]), acc, 0,
+                                                      0, 0);
+    }
+    if (pair >= 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = r0 + 4 * g4 + r;
+        if (row < NR) {
+          if (UP) {
+            const float v = fmaxf(acc[r], 0.f);
+            reinterpret_cast<bf16_t*>(dst)[(long)pair * NR + row] =
+                f2us(v * v);
+          } else {
+            reinterpret_cast<float*>(dst)[(long)pair * NR + row] = acc[r];
+          }
+        }
+      }
+    }
+  }
+}
+
 // out, h [T, W]; ids [T] int32; table [vocab, top] int32; w_up [E, ff, W];
 // w_down [E, W, ff].
 void table_moe(torch::Tensor out, torch::Tensor h, torch::Tensor ids,
@@ -107,21 +323,82 @@ void table_moe(torch::Tensor out, torch::Tensor h, torch::Tensor ids,
   auto act = torch::empty({rows * top, (long)ff}, h.options());
   auto stream = c10::hip::getCurrentHIPStream().stream();
   const int per_block = 4 * MOE_ROWS_PER_WAVE;
+  const long pairs = rows * top;
+  // expert-major kernels: vector loads need whole 16-byte chunks
+  const bool small = pairs <= MOE_MAX_PAIRS;
+  const bool up_major = small && W % 8 == 0 && aligned16(h.data_ptr()) &&
+                        aligned16(w_up.data_ptr());
+  const bool down_major = small && ff % 8 == 0 && aligned16(act.data_ptr()) &&
+                          aligned16(w_down.data_ptr());
+  torch::Tensor part;
+  if (down_major || (up_major && W / 8 > MOE_SEG * WAVE))
+    part = torch::empty({pairs, (long)std::max(W, ff)},
+                        h.options().dtype(torch::kFloat32));
+  float* pp = part.defined() ? part.data_ptr<float>() : nullptr;
+  // bf16 rows of whole 128-element blocks go to the matrix cores
+  const bool bf = is_bf16(h);
+  const bool up_mfma = up_major && bf && W % 128 == 0;
+  const bool down_mfma = down_major && bf && ff % 128 == 0;
+  const bf16_t* hb = reinterpret_cast<const bf16_t*>(h.data_ptr());
+  const bf16_t* ab = reinterpret_cast<const bf16_t*>(act.data_ptr());
+  if (up_mfma)
+    table_moe_mfma_kernel<true><<<
+        dim3((unsigned)E, (unsigned)((ff + 63) / 64)), 256, 0, stream>>>(
+        act.data_ptr(), hb, ids.data_ptr<int>(), table.data_ptr<int>(),
+        reinterpret_cast<const bf16_t*>(w_up.data_ptr()), ff, W, top, vocab,
+        (int)pairs);
+  if (down_mfma) {
+    table_moe_mfma_kernel<false><<<
+        dim3((unsigned)E, (unsigned)((W + 63) / 64)), 256, 0, stream>>>(
+        pp, ab, ids.data_ptr<int>(), table.data_ptr<int>(),
+        reinterpret_cast<const bf16_t*>(w_down.data_ptr()), W, ff, top, vocab,
+        (int)pairs);
+    const long total = rows * W;
+    table_moe_mean_kernel<bf16_t><<<dim3((unsigned)((total + 255) / 256)), 256,
+                                    0, stream>>>(
+        reinterpret_cast<bf16_t*>(out.data_ptr()), pp, total, W, top);
+  }
   KK_DISPATCH_ACT(h, {
-    table_moe_up_kernel<T><<<dim3((unsigned)(rows * top),
-                                  (unsigned)((ff + per_block - 1) / per_block)),
-                             256, (size_t)W * 4, stream>>>(
-        reinterpret_cast<T*>(act.data_ptr()),
-        reinterpret_cast<const T*>(h.data_ptr()), ids.data_ptr<int>(),
-        table.data_ptr<int>(), reinterpret_cast<const T*>(w_up.data_ptr()), W,
-        ff, top, vocab);
-    table_moe_down_kernel<T><<<dim3((unsigned)rows,
-                                    (unsigned)((W + per_block - 1) / per_block)),
-                               256, (size_t)top * ff * 4, stream>>>(
-        reinterpret_cast<T*>(out.data_ptr()),
-        reinterpret_cast<const T*>(act.data_ptr()), ids.data_ptr<int>(),
-        table.data_ptr<int>(), reinterpret_cast<const T*>(w_down.data_ptr()),
-        W, ff, top, vocab);
+    if (up_mfma) {
+    } else if (up_major)
+      table_moe_up_expert_kernel<T><<<
+          dim3((unsigned)E, (unsigned)((ff + per_block - 1) / per_block)), 256,
+          0, stream>>>(
+          reinterpret_cast<T*>(act.data_ptr()), pp,
+          reinterpret_cast<const T*>(h.data_ptr()), ids.data_ptr<int>(),
+          table.data_ptr<int>(), reinterpret_cast<const T*>(w_up.data_ptr()),
+          W, ff, top, vocab, (int)pairs);
+    else
+      table_moe_up_kernel<T><<<
+          dim3((unsigned)(rows * top),
+               (unsigned)((ff + per_block - 1) / per_block)),
+          256, (size_t)W * 4, stream>>>(
+          reinterpret_cast<T*>(act.data_ptr()),
+          reinterpret_cast<const T*>(h.data_ptr()), ids.data_ptr<int>(),
+          table.data_ptr<int>(), reinterpret_cast<const T*>(w_up.data_ptr()),
+          W, ff, top, vocab);
+    if (down_mfma) {
+    } else if (down_major) {
+      table_moe_down_expert_kernel<T><<<
+          dim3((unsigned)E, (unsigned)((W + per_block - 1) / per_block)), 256,
+          0, stream>>>(
+          pp, reinterpret_cast<const T*>(act.data_ptr()), ids.data_ptr<int>(),
+          table.data_ptr<int>(),
+          reinterpret_cast<const T*>(w_down.data_ptr()), W, ff, top, vocab,
+          (int)pairs);
+      const long total = rows * W;
+      table_moe_mean_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0,
+                                 stream>>>(
+          reinterpret_cast<T*>(out.data_ptr()), pp, total, W, top);
+    } else {
+      table_moe_down_kernel<T><<<
+          dim3((unsigned)rows, (unsigned)((W + per_block - 1) / per_block)),
+          256, (size_t)top * ff * 4, stream>>>(
+          reinterpret_cast<T*>(out.data_ptr()),
+          reinterpret_cast<const T*>(act.data_ptr()), ids.data_ptr<int>(),
+          table.data_ptr<int>(),
+          reinterpret_cast<const T*>(w_down.data_ptr()), W, ff, top, vocab);
+    }
   });
   HIP_CHECK_KERNEL();
 }

@@ -620,7 +620,7 @@ def case_op_activations(device, dtype):
     _close(out, want, dtype, "head gate")
 
 
-def case_op_table_moe(device, dtype, E=5, top=2, W=24, ff=13, V=11):
+def case_op_table_moe(device, dtype, E=5, top=2, W=24, ff=13, V=11, rows=9):
     from kukeon_amd import ops
     g = torch.Generator().manual_seed(E * 10 + top)
     act = _act(dtype)
@@ -630,9 +630,9 @@ def case_op_table_moe(device, dtype, E=5, top=2, W=24, ff=13, V=11):
               for e in range(E)})
     t["table"] = torch.stack([torch.randperm(E, generator=g)[:top]
                               for _ in range(V)]).to(torch.int32)
-    ids = torch.randint(0, V, (9,), generator=g)
-    h = torch.randn(9, W, generator=g).to(act)
-    out = torch.empty(9, W, dtype=act, device=device)
+    ids = torch.randint(0, V, (rows,), generator=g)
+    h = torch.randn(rows, W, generator=g).to(act)
+    out = torch.empty(rows, W, dtype=act, device=device)
     ops.table_moe(out, h.to(device), ids.to(torch.int32).to(device),
                   t["table"].to(device),
                   torch.stack([t[f"e{e}.up"] for e in range(E)]).to(device),

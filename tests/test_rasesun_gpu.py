@@ -54,6 +54,16 @@ def test_op_activations(dtype):
 def test_op_table_moe(top, dtype):
     cases.case_op_table_moe(DEV, dtype, top=top)
     cases.case_op_table_moe(DEV, dtype, E=7, top=top, W=136, ff=70, V=19)
+    # whole 16-byte chunks both ways: the expert-major kernels
+    cases.case_op_table_moe(DEV, dtype, E=7, top=top, W=136, ff=72, V=19)
+    # whole 128-element blocks: the matrix-core kernels in bf16; an expert
+    # with more pairs than one tile holds, row counts that end inside a tile
+    cases.case_op_table_moe(DEV, dtype, E=3, top=top, W=256, ff=136,
+                            V=19, rows=45)
+    cases.case_op_table_moe(DEV, dtype, E=6, top=top, W=128, ff=384, V=8,
+                            rows=5)
+    # rows longer than one register segment
+    cases.case_op_table_moe(DEV, dtype, E=4, top=top, W=8200, ff=16, V=9)
 
 
 @BOTH
