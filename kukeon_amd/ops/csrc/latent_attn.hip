@@ -96,14 +96,6 @@ void latent_kv_append(torch::Tensor cq_out, torch::Tensor cache,
   TORCH_CHECK(block_table.dim() == 2);
   if (rows == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
-#define KK_ARGS reinterpret_cast<T*>(out.data_ptr()),                        \
-        reinterpret_cast<const T*>(q_abs.data_ptr()),                        \
-        reinterpret_cast<const T*>(q.data_ptr()), (long)q.stride(0),         \
-        reinterpret_cast<const T*>(cache.data_ptr()), cs.data_ptr<float>(),  \
-        (int)cs.size(0), (int)cs.size(1), positions.data_ptr<int>(),         \
-        row_seq.data_ptr<int>(), block_table.data_ptr<int>(),                \
-        (int)block_table.size(1), rows, (int)H, (int)dn, (int)dr, R,         \
-        (int)cache.size(2), (int)window, (float)scale
   KK_DISPATCH_ACT(proj, {
     latent_kv_append_kernel<T><<<dim3((unsigned)rows), 256, 0, stream>>>(
         reinterpret_cast<T*>(cq_out.data_ptr()),
@@ -257,6 +249,158 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
   }
 }
 
+// Vector form of the same walk: rows of whole 16-byte chunks, a latent of
+// 8 * 2^k entries. Scores: thread j reads its key row in 16-byte pieces.
+// Weighted sum: R/8 threads cover one latent row (8 entries each) and the
+// 256 / (R/8) thread groups take every NG-th key of the chunk; the groups'
+// partial sums meet in LDS at the end, added in group order.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_attention_vec_kernel(
+    T* __restrict__ out, const T* __restrict__ q_abs, const T* __restrict__ q,
+    long ldq, const T* __restrict__ cache, const float* __restrict__ cs,
+    int cs_rows, int dims, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ block_table,
+    int max_blocks, long rows, int H, int dn, int dr, int R, int BS,
+    int window, float scale) {
+  extern __shared__ float sm[];
+  const int KW = R + dr;
+  float* sq = sm;                          // [HB][KW]
+  float* sc = sq + LAT_HB * KW;            // [HB][CH]
+  float* part = sc + LAT_HB * LAT_CH;      // [NG][HB][R] = 256 * 32 floats
+  __shared__ float red[32];
+  __shared__ long srow[LAT_CH];
+  const long r = blockIdx.x;
+  const int h0 = blockIdx.y * LAT_HB;
+  const int tid = threadIdx.x;
+  const int p = positions[r];
+  if (p < 0) {
+    for (int hb = 0; hb < LAT_HB && h0 + hb < H; ++hb)
+      for (int d = tid; d < R; d += blockDim.x)
+        stf(out + ((long)(h0 + hb) * rows + r) * R + d, 0.f);
+    return;
+  }
+  const int s = row_seq[r];
+  const int pp = p < cs_rows ? p : cs_rows - 1;
+  const float* ang = cs + (long)pp * dims;
+  const int half = dims / 2;
+  for (int i = tid; i < LAT_HB * KW; i += blockDim.x) {
+    const int hb = i / KW, d = i - hb * KW;
+    const int h = h0 + hb;
+    float v = 0.f;
+    if (h < H) {
+      if (d < R) {
+        v = ldf(q_abs + ((long)h * rows + r) * R + d);
+      } else {
+        const int e = d - R;
+        const T* qr = q + r * ldq + (long)h * (dn + dr) + dn;
+        v = ldf(qr + e);
+        if (e < dims) {
+          const float other = ldf(qr + (e ^ 1));
+          const float c = ang[e >> 1], sn = ang[half + (e >> 1)];
+          v = (e & 1) ? fmaf(v, c, other * sn) : fmaf(v, c, -other * sn);
+        }
+      }
+    }
+    sq[i] = v;
+  }
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int nkeys = p - lo + 1;
+  const int per_row = R / 8;               // threads that cover one latent
+  const int NG = 256 / per_row;
+  const int dg = tid % per_row;
+  const int kg = tid / per_row;
+  float m[LAT_HB], l[LAT_HB], acc[LAT_HB][8];
+#pragma unroll
+  for (int hb = 0; hb < LAT_HB; ++hb) {
+    m[hb] = -INFINITY;
+    l[hb] = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[hb][k] = 0.f;
+  }
+  const int* bt = block_table + (long)s * max_blocks;
+  const int nchunks8 = KW / 8;
+  for (int c0 = 0; c0 < nkeys; c0 += LAT_CH) {
+    const int cn = min(LAT_CH, nkeys - c0);
+    __syncthreads();
+    float sv[LAT_HB];
+#pragma unroll
+    for (int hb = 0; hb < LAT_HB; ++hb) sv[hb] = -INFINITY;
+    if (tid < cn) {
+      const int j = lo + c0 + tid;
+      const long base = ((long)bt[j / BS] * BS + j % BS) * KW;
+      srow[tid] = base;
+      const T* kr = cache + base;
+      float a[LAT_HB];
+#pragma unroll
+      for (int hb = 0; hb < LAT_HB; ++hb) a[hb] = 0.f;
+#pragma unroll 4
+      for (int d8 = 0; d8 < nchunks8; ++d8) {
+        Raw8<T> kv;
+        kv.load(kr + d8 * 8);
+#pragma unroll
+        for (int hb = 0; hb < LAT_HB; ++hb) {
+          const float* qh = sq + hb * KW + d8 * 8;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) a[hb] = fmaf(qh[k], kv.get(k), a[hb]);
+        }
+      }
+#pragma unroll
+      for (int hb = 0; hb < LAT_HB; ++hb) sv[hb] = a[hb] * scale;
+    }
+    float alpha[LAT_HB];
+#pragma unroll
+    for (int hb = 0; hb < LAT_HB; hb += 2) {
+      const float2 mx = block_max2(sv[hb], sv[hb + 1], red);
+      const float m0 = fmaxf(m[hb], mx.x), m1 = fmaxf(m[hb + 1], mx.y);
+      alpha[hb] = __expf(m[hb] - m0);
+      alpha[hb + 1] = __expf(m[hb + 1] - m1);
+      m[hb] = m0;
+      m[hb + 1] = m1;
+      const float w0 = tid < cn ? __expf(sv[hb] - m0) : 0.f;
+      const float w1 = tid < cn ? __expf(sv[hb + 1] - m1) : 0.f;
+      sc[hb * LAT_CH + tid] = w0;
+      sc[(hb + 1) * LAT_CH + tid] = w1;
+      const float2 su = block_sum2(w0, w1, red);
+      l[hb] = l[hb] * alpha[hb] + su.x;
+      l[hb + 1] = l[hb + 1] * alpha[hb + 1] + su.y;
+    }
+#pragma unroll
+    for (int hb = 0; hb < LAT_HB; ++hb)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc[hb][k] *= alpha[hb];
+#pragma unroll 4
+    for (int jj = kg; jj < cn; jj += NG) {
+      Raw8<T> cv;
+      cv.load(cache + srow[jj] + dg * 8);
+#pragma unroll
+      for (int hb = 0; hb < LAT_HB; ++hb) {
+        const float w = sc[hb * LAT_CH + jj];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[hb][k] = fmaf(w, cv.get(k), acc[hb][k]);
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int hb = 0; hb < LAT_HB; ++hb)
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      part[((long)kg * LAT_HB + hb) * R + dg * 8 + k] = acc[hb][k];
+  __syncthreads();
+  for (int i = tid; i < LAT_HB * R; i += blockDim.x) {
+    const int hb = i / R, d = i - hb * R;
+    const int h = h0 + hb;
+    if (h >= H) continue;
+    float sum = 0.f;
+    for (int g = 0; g < NG; ++g) sum += part[((long)g * LAT_HB + hb) * R + d];
+    // l is the same in every thread; pick it by a uniform chain
+    float lh = l[0];
+#pragma unroll
+    for (int x = 1; x < LAT_HB; ++x) lh = hb == x ? l[x] : lh;
+    stf(out + ((long)h * rows + r) * R + d, sum / lh);
+  }
+}
+
 // out, q_abs [H, rows, R] contiguous; q [rows, >= H*(dn+dr)] (stride(1) ==
 // 1); cache [blocks, 1, BS, R+dr]; cs [positions, dims] fp32.
 void latent_attention(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q,
@@ -291,8 +435,24 @@ void latent_attention(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q,
   TORCH_CHECK(lds <= 60 * 1024, "latent_attention: queries do not fit LDS");
   auto stream = c10::hip::getCurrentHIPStream().stream();
   dim3 grid((unsigned)rows, (unsigned)((H + LAT_HB - 1) / LAT_HB));
+  // vector form: whole 16-byte chunks and a latent of 8 * 2^k entries
+  const int per_row = R / 8;
+  const bool vec = R % 8 == 0 && dr % 8 == 0 && per_row >= 1 &&
+                   per_row <= 256 && (per_row & (per_row - 1)) == 0 &&
+                   aligned16(cache.data_ptr());
+  const size_t lds_vec = lds + (size_t)256 * LAT_HB * 8 * 4;
+#define KK_ARGS reinterpret_cast<T*>(out.data_ptr()),                        \
+        reinterpret_cast<const T*>(q_abs.data_ptr()),                        \
+        reinterpret_cast<const T*>(q.data_ptr()), (long)q.stride(0),         \
+        reinterpret_cast<const T*>(cache.data_ptr()), cs.data_ptr<float>(),  \
+        (int)cs.size(0), (int)cs.size(1), positions.data_ptr<int>(),         \
+        row_seq.data_ptr<int>(), block_table.data_ptr<int>(),                \
+        (int)block_table.size(1), rows, (int)H, (int)dn, (int)dr, R,         \
+        (int)cache.size(2), (int)window, (float)scale
   KK_DISPATCH_ACT(q, {
-    if (R <= 256)
+    if (vec && lds_vec <= 60 * 1024)
+      latent_attention_vec_kernel<T><<<grid, 256, lds_vec, stream>>>(KK_ARGS);
+    else if (R <= 256)
       latent_attention_kernel<T, 1><<<grid, 256, lds, stream>>>(KK_ARGS);
     else if (R <= 512)
       latent_attention_kernel<T, 2><<<grid, 256, lds, stream>>>(KK_ARGS);

@@ -110,8 +110,6 @@ void residual_add_rmsnorm(torch::Tensor x, torch::Tensor a, torch::Tensor bias,
                                aligned16(a.data_ptr()))) &&
                    (!has_b || aligned16(bias.data_ptr()));
   if (vec) {
-  #define KK_ARGS x.data_ptr<float>(), yp, (long)y.stride(0),                \
-        post_w.data_ptr<float>(), w.data_ptr<float>(), (float)eps, op, W
   KK_DISPATCH_ACT(out, {
       const T* ap = has_a ? reinterpret_cast<const T*>(a.data_ptr()) : nullptr;
       const long lda = has_a ? a.stride(0) : 0;
@@ -259,6 +257,8 @@ void postnorm_residual_rmsnorm(torch::Tensor x, torch::Tensor y,
                    aligned16(out.data_ptr()) && aligned16(w.data_ptr()) &&
                    aligned16(post_w.data_ptr()) && y.stride(0) % 8 == 0 &&
                    aligned16(y.data_ptr());
+#define KK_ARGS x.data_ptr<float>(), yp, (long)y.stride(0),                \
+        post_w.data_ptr<float>(), w.data_ptr<float>(), (float)eps, op, W
   KK_DISPATCH_ACT(out, {
     const T* yp = reinterpret_cast<const T*>(y.data_ptr());
     T* op = reinterpret_cast<T*>(out.data_ptr());

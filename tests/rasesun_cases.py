@@ -74,6 +74,15 @@ CONFIGS = {
         layer(latent(heads=5, dim=16, rot_dim=8, vdim=12, q_rank=32,
                      kv_rank=300, window=290), dense(64)),
     ], width=64, vocab=61, scale=1.0, eps=1e-3, softcap=30.0),
+    # every width a multiple of 8 or 128: the vector and matrix-core forms
+    # of the kernels (16-byte loads, expert tiles), six heads on a head
+    # group of four
+    "aligned": lambda: config([
+        layer(ssm(heads=2, vdim=32, state=16, groups=1, conv=4,
+                  norm_groups=2), moe(4, 2, 128)),
+        layer(latent(heads=6, dim=16, rot_dim=8, vdim=16, q_rank=24,
+                     kv_rank=32, window=20), moe(3, 1, 128)),
+    ], width=128, vocab=50, loop=(0, 2, 2)),
     # the whole stack looped, attention first, window of one, one tap,
     # no embedding scale, no soft cap
     "looped": lambda: _looped(),

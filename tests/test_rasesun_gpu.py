@@ -78,6 +78,11 @@ def test_op_latent_attention(dtype):
     # workgroup
     cases.case_op_latent_attention(DEV, dtype, ctx=700, BS=16, H=3, R=300,
                                    dr=8, window=600)
+    # whole 16-byte chunks: the vector form, one and several key chunks
+    cases.case_op_latent_attention(DEV, dtype, ctx=300, BS=16, H=5, R=64,
+                                   dr=8, window=40)
+    cases.case_op_latent_attention(DEV, dtype, ctx=700, BS=8, H=9, R=512,
+                                   dr=64, window=600)
 
 
 @BOTH
@@ -104,7 +109,7 @@ def test_portions(sizes, dtype):
 
 
 @BOTH
-@pytest.mark.parametrize("name", ["hybrid", "wide", "looped"])
+@pytest.mark.parametrize("name", ["hybrid", "wide", "looped", "aligned"])
 def test_unequal_batch(name, dtype):
     cases.case_batch(name, DEV, dtype)
 
