@@ -401,6 +401,203 @@ __global__ __launch_bounds__(256) void latent_attention_vec_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Matrix-core form for prompt portions (bf16). One wave owns (row, 16 heads)
+// and walks the row's window 16 keys at a time; tiles start at multiples of
+// 16 in absolute position, so a row's sums do not depend on where its portion
+// began. No barriers: the two waves of a workgroup are independent and each
+// has its own LDS area.
+//   scores  S^T[key, head] = K[key, :] . Q[head, :]   v_mfma_f32_16x16x32_bf16
+//           A = cache rows straight from memory (lane = key, 8 entries of the
+//           row per k block), B = the query fragments held in registers.
+//   softmax per head in fp32: a lane holds 4 keys of one head, two exchanges
+//           across the 4 lane groups complete the maximum and the sum.
+//   sum     O^T[d, head] += C^T[d, key] P[key, head]  v_mfma_f32_16x16x16bf16_1k
+//           The score layout is already the B layout of P. The latent part
+//           of the key tile is written to LDS as it arrives and read back
+//           transposed as the A operand. P enters as hi + lo (two products)
+//           so that the weights keep fp32 accuracy.
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short lat_bf16x8_v;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short lat_bf16x4_v;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float lat_f32x4_v;
+
+DEV_INLINE lat_bf16x8_v lat_frag8(const uint4& v) {
+  return __builtin_bit_cast(lat_bf16x8_v, v);
+}
+DEV_INLINE lat_bf16x4_v lat_frag4(unsigned short a, unsigned short b,
+                                  unsigned short c, unsigned short d) {
+  lat_bf16x4_v v;
+  v[0] = (short)a; v[1] = (short)b; v[2] = (short)c; v[3] = (short)d;
+  return v;
+}
+
+template <int R, int DR>
+__global__ __launch_bounds__(128) void latent_attention_mfma_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q_abs,
+    const bf16_t* __restrict__ q, long ldq, const bf16_t* __restrict__ cache,
+    const float* __restrict__ cs, int cs_rows, int dims,
+    const int* __restrict__ positions, const int* __restrict__ row_seq,
+    const int* __restrict__ block_table, int max_blocks, long rows, int H,
+    int dn, int BS, int window, float scale, int HT) {
+  constexpr int KW = R + DR, KST = KW / 32, VST = R / 32, NDT = R / 16;
+  constexpr int LDV = R + 8;               // padded LDS row, 16-byte aligned
+  extern __shared__ unsigned short lat_lds[];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int rc = lane & 15;
+  const int g4 = lane >> 4;
+  const long unit = (long)blockIdx.x * 2 + wave;
+  if (unit >= rows * HT) return;
+  const long r = unit / HT;
+  const int h = (int)(unit - r * HT) * 16 + rc;
+  unsigned short* vl = lat_lds + wave * 16 * LDV;
+  bf16_t* orow = out + ((long)(h < H ? h : 0) * rows + r) * R + 4 * g4;
+  const int p = positions[r];
+  if (p < 0) {
+    if (h < H)
+      for (int dt = 0; dt < NDT; ++dt)
+        *reinterpret_cast<uint2*>(orow + dt * 16) = uint2{0u, 0u};
+    return;
+  }
+  const int s = row_seq[r];
+  // ---- query fragments: latent part, then the rotated part ----
+  uint4 qf[KST];
+#pragma unroll
+  for (int st = 0; st < VST; ++st)
+    qf[st] = h < H ? *reinterpret_cast<const uint4*>(
+                         q_abs + ((long)h * rows + r) * R + st * 32 + g4 * 8)
+                   : uint4{0u, 0u, 0u, 0u};
+  {
+    const int pp = p < cs_rows ? p : cs_rows - 1;
+    const float* ang = cs + (long)pp * dims;
+    const int half = dims / 2;
+#pragma unroll
+    for (int st = 0; st < DR / 32; ++st) {
+      uint4 v = uint4{0u, 0u, 0u, 0u};
+      if (h < H) {
+        float f[8];
+        ld8(q + r * ldq + (long)h * (dn + DR) + dn + st * 32 + g4 * 8, f);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int e0 = st * 32 + g4 * 8 + 2 * i;
+          if (e0 < dims) {
+            const float c = ang[e0 >> 1], sn = ang[half + (e0 >> 1)];
+            const float a = f[2 * i], b = f[2 * i + 1];
+            f[2 * i] = fmaf(a, c, -b * sn);
+            f[2 * i + 1] = fmaf(b, c, a * sn);
+          }
+        }
+        v = pack_bf16x8(f);
+      }
+      qf[VST + st] = v;
+    }
+  }
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int* bt = block_table + (long)s * max_blocks;
+  lat_f32x4_v o[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) o[dt] = lat_f32x4_v{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  for (int j0 = lo & ~15; j0 <= p; j0 += 16) {
+    // the lane's key, kept inside the visible range for the loads
+    int jc = j0 + rc;
+    jc = jc < lo ? lo : (jc > p ? p : jc);
+    const bf16_t* kr =
+        cache + ((long)bt[jc / BS] * BS + jc % BS) * KW + g4 * 8;
+    lat_f32x4_v sacc = {0.f, 0.f, 0.f, 0.f};
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int st = 0; st < KST; ++st) {
+      const uint4 a = *reinterpret_cast<const uint4*>(kr + st * 32);
+      sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lat_frag8(a),
+                                                     lat_frag8(qf[st]), sacc,
+                                                     0, 0, 0);
+      if (st < VST)
+        *reinterpret_cast<uint4*>(vl + rc * LDV + st * 32 + g4 * 8) = a;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // ---- online softmax: lane = (head rc, keys j0 + 4 g4 + i) ----
+    float sv[4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = j0 + 4 * g4 + i;
+      sv[i] = (j >= lo && j <= p) ? sacc[i] * scale : -INFINITY;
+      tmax = fmaxf(tmax, sv[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float mn = fmaxf(m, tmax);       // every tile holds a visible key
+    const float alpha = (m == -INFINITY) ? 0.f : __expf(m - mn);
+    m = mn;
+    float psum = 0.f;
+    unsigned short ph[4], pl[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float w = (sv[i] == -INFINITY) ? 0.f : __expf(sv[i] - mn);
+      psum += w;
+      ph[i] = f2us(w);
+      pl[i] = f2us(w - us2f(ph[i]));
+    }
+    psum += __shfl_xor(psum, 16, WAVE);
+    psum += __shfl_xor(psum, 32, WAVE);
+    l = l * alpha + psum;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) o[dt] *= alpha;
+    }
+    const lat_bf16x4_v phi = lat_frag4(ph[0], ph[1], ph[2], ph[3]);
+    const lat_bf16x4_v plo = lat_frag4(pl[0], pl[1], pl[2], pl[3]);
+    const unsigned short* vp = vl + (4 * g4) * LDV + rc;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      const lat_bf16x4_v a =
+          lat_frag4(vp[dt * 16], vp[dt * 16 + LDV], vp[dt * 16 + 2 * LDV],
+                    vp[dt * 16 + 3 * LDV]);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, phi, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, plo, o[dt], 0, 0, 0);
+    }
+  }
+  if (h >= H) return;
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    const unsigned int w0 = (unsigned int)f2us(o[dt][0] * inv) |
+                            ((unsigned int)f2us(o[dt][1] * inv) << 16);
+    const unsigned int w1 = (unsigned int)f2us(o[dt][2] * inv) |
+                            ((unsigned int)f2us(o[dt][3] * inv) << 16);
+    *reinterpret_cast<uint2*>(orow + dt * 16) = uint2{w0, w1};
+  }
+}
+
+template <int R, int DR>
+static void launch_latent_mfma(torch::Tensor& out, torch::Tensor& q_abs,
+                               torch::Tensor& q, torch::Tensor& cache,
+                               torch::Tensor& cs, torch::Tensor& positions,
+                               torch::Tensor& row_seq,
+                               torch::Tensor& block_table, long rows, int H,
+                               int dn, int window, float scale,
+                               hipStream_t stream) {
+  const int HT = (H + 15) / 16;
+  const long units = rows * HT;
+  const size_t lds = (size_t)2 * 16 * (R + 8) * sizeof(unsigned short);
+  latent_attention_mfma_kernel<R, DR>
+      <<<dim3((unsigned)((units + 1) / 2)), 128, lds, stream>>>(
+          reinterpret_cast<bf16_t*>(out.data_ptr()),
+          reinterpret_cast<const bf16_t*>(q_abs.data_ptr()),
+          reinterpret_cast<const bf16_t*>(q.data_ptr()), (long)q.stride(0),
+          reinterpret_cast<const bf16_t*>(cache.data_ptr()),
+          cs.data_ptr<float>(), (int)cs.size(0), (int)cs.size(1),
+          positions.data_ptr<int>(), row_seq.data_ptr<int>(),
+          block_table.data_ptr<int>(), (int)block_table.size(1), rows, H, dn,
+          (int)cache.size(2), window, scale, HT);
+}
+
+// sizes the matrix-core form serves
+bool latent_attention_mfma_supported(int64_t R, int64_t dr) {
+  return (R == 128 || R == 256 || R == 512) && (dr == 32 || dr == 64);
+}
+
 // out, q_abs [H, rows, R] contiguous; q [rows, >= H*(dn+dr)] (stride(1) ==
 // 1); cache [blocks, 1, BS, R+dr]; cs [positions, dims] fp32.
 void latent_attention(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q,
@@ -435,6 +632,26 @@ void latent_attention(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q,
   TORCH_CHECK(lds <= 60 * 1024, "latent_attention: queries do not fit LDS");
   auto stream = c10::hip::getCurrentHIPStream().stream();
   dim3 grid((unsigned)rows, (unsigned)((H + LAT_HB - 1) / LAT_HB));
+  // prompt portions in bf16 at the served sizes: the matrix cores. Few rows
+  // (a decode step) leave them idle, so those stay with the vector form.
+  if (is_bf16(q) && latent_attention_mfma_supported(R, dr) && dn % 8 == 0 &&
+      q.stride(0) % 8 == 0 && aligned16(q.data_ptr()) &&
+      aligned16(cache.data_ptr()) && aligned16(q_abs.data_ptr()) &&
+      aligned16(out.data_ptr()) && rows * ((H + 15) / 16) >= 512) {
+#define KK_MFMA(RR, DD)                                                      \
+  launch_latent_mfma<RR, DD>(out, q_abs, q, cache, cs, positions, row_seq,   \
+                             block_table, rows, (int)H, (int)dn, (int)window, \
+                             (float)scale, stream)
+    if (R == 128 && dr == 32) KK_MFMA(128, 32);
+    else if (R == 128) KK_MFMA(128, 64);
+    else if (R == 256 && dr == 32) KK_MFMA(256, 32);
+    else if (R == 256) KK_MFMA(256, 64);
+    else if (R == 512 && dr == 32) KK_MFMA(512, 32);
+    else KK_MFMA(512, 64);
+#undef KK_MFMA
+    HIP_CHECK_KERNEL();
+    return;
+  }
   // vector form: whole 16-byte chunks and a latent of 8 * 2^k entries
   const int per_row = R / 8;
   const bool vec = R % 8 == 0 && dr % 8 == 0 && per_row >= 1 &&

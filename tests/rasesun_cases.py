@@ -83,6 +83,14 @@ CONFIGS = {
         layer(latent(heads=6, dim=16, rot_dim=8, vdim=16, q_rank=24,
                      kv_rank=32, window=20), moe(3, 1, 128)),
     ], width=128, vocab=50, loop=(0, 2, 2)),
+    # a latent of 128 with a rotated part of 32: the sizes of the
+    # matrix-core attention kernel, which long portions take
+    "tiles": lambda: config([
+        layer(ssm(heads=2, vdim=16, state=8, groups=2, conv=2,
+                  norm_groups=1), None),
+        layer(latent(heads=3, dim=8, rot_dim=32, rot_dims=12, vdim=8,
+                     q_rank=16, kv_rank=128, window=50), dense(48)),
+    ], width=48, vocab=40),
     # the whole stack looped, attention first, window of one, one tap,
     # no embedding scale, no soft cap
     "looped": lambda: _looped(),
@@ -402,6 +410,25 @@ def case_grouped_experts(device, dtype):
     got = run_schedule(eng, prompts, sched)
     for i in range(2):
         check(got[i], want[i], dtype, f"token by token, request {i}")
+
+
+def case_long_portions(device, dtype):
+    """Portions long enough for the matrix-core attention kernel beside
+    short ones and single tokens that take the other forms."""
+    cfg = CONFIGS["tiles"]()
+    W = weights(cfg, 13)
+    prompts = [tokens(cfg, n, 80 + n) for n in (560, 70)]
+    want = [oracle.forward(cfg, W, p) for p in prompts]
+    eng = make_engine(cfg, W, device, dtype, blocks=48, block_size=16,
+                      max_len=640)
+    got = run_schedule(eng, prompts, [[(0, 560), (1, 69)], [(1, 1)]])
+    for i in range(2):
+        check(got[i], want[i], dtype, f"whole, request {i}")
+    got = run_schedule(eng, prompts,
+                       [[(0, 21)], [(0, 530), (1, 2)], [(0, 1), (1, 68)],
+                        [(0, 8)]])
+    for i in range(2):
+        check(got[i], want[i], dtype, f"portions, request {i}")
 
 
 def case_greedy(device, dtype, graphs=False):
@@ -751,6 +778,9 @@ def case_op_latent_attention(device, dtype, ctx=300, BS=16, H=5, R=24, dr=6,
         return out.permute(1, 0, 2)
 
     _close(run(rows), want[rows], dtype, "prompt rows", scale=1.0)
+    _close(run(list(range(ctx))), want, dtype, "every row", scale=1.0)
+    _close(run(list(range(37, ctx))), want[37:], dtype, "a portion's rows",
+           scale=1.0)
     for r in probes + [0, window]:
         _close(run([r]), want[[r]], dtype, f"decoded row {r}", scale=1.0)
     out = run(rows[:3], [rows[0], -1, rows[2]])

@@ -50,6 +50,10 @@ def test_long_portions_sort_rows_by_expert():
     cases.case_grouped_experts(DEV, DT)
 
 
+def test_long_portions():
+    cases.case_long_portions(DEV, DT)
+
+
 def test_greedy_generation():
     cases.case_greedy(DEV, DT)
 

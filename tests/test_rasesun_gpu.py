@@ -83,6 +83,11 @@ def test_op_latent_attention(dtype):
                                    dr=8, window=40)
     cases.case_op_latent_attention(DEV, dtype, ctx=700, BS=8, H=9, R=512,
                                    dr=64, window=600)
+    # sizes of the matrix-core form; two head tiles, the second partly filled
+    cases.case_op_latent_attention(DEV, dtype, ctx=600, BS=16, H=20, R=128,
+                                   dr=32, window=100)
+    cases.case_op_latent_attention(DEV, dtype, ctx=520, BS=4, H=3, R=256,
+                                   dr=64, window=33)
 
 
 @BOTH
@@ -132,6 +137,11 @@ def test_long_decode(dtype):
 @BOTH
 def test_window_longer_than_a_key_chunk(dtype):
     cases.case_window_chunks(DEV, dtype)
+
+
+@BOTH
+def test_long_portions_on_the_matrix_cores(dtype):
+    cases.case_long_portions(DEV, dtype)
 
 
 @BOTH
