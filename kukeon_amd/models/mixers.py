@@ -111,7 +111,7 @@ class StateSpaceMixer(nn.Module):
 
     def state_shape(self):
         m = self.m
-        return [(m.conv - 1, m.conv_channels), (m.heads, m.state, m.vdim)]
+        return [(m.conv - 1, m.conv_channels), (m.heads, m.vdim, m.state)]
 
     def forward(self, h: torch.Tensor, cache, state, meta) -> torch.Tensor:
         m = self.m

@@ -42,6 +42,48 @@ __global__ __launch_bounds__(256) void conv_act_kernel(
   stf(out + r * (long)C + c, acc);
 }
 
+// Vector form: 8 consecutive channels per thread, every tap one 16-byte (bf16)
+// or 32-byte (fp32) load; the same sums in the same order.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_act_vec_kernel(
+    T* __restrict__ out, const T* __restrict__ proj, long ldp, long col0,
+    const float* __restrict__ cw, const float* __restrict__ bias,
+    const float* __restrict__ state, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ cu_rows,
+    const int* __restrict__ state_slots, int C, int taps, int act) {
+  const long r = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (c >= C) return;
+  const int p = positions[r];
+  if (p < 0) return;
+  const int s = row_seq[r];
+  const long row0 = cu_rows[s];
+  const int i = (int)(r - row0);
+  const int back = taps - 1;
+  const float* st = state + (long)state_slots[s] * back * C;
+  float acc[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) acc[k] = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int src = i - back + j;
+    if (p - back + j < 0) continue;
+    float u[8], w[8];
+    if (src >= 0) ld8(proj + (row0 + src) * ldp + col0 + c, u);
+    else ld8(st + (long)(back + src) * C + c, u);
+    ld8(cw + (long)j * C + c, w);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = fmaf(w[k], u[k], acc[k]);
+  }
+  float b[8];
+  ld8(bias + c, b);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    acc[k] += b[k];
+    if (act == 1) acc[k] = acc[k] / (1.0f + __expf(-acc[k]));
+  }
+  st8(out + r * (long)C + c, acc);
+}
+
 // out [rows, C] contiguous; proj [rows, ld] (stride(1) == 1) read at
 // columns col0 .. col0+C-1; cw [taps, C], bias [C] fp32; state
 // [slots, taps-1, C] fp32.
@@ -68,6 +110,25 @@ void conv_act(torch::Tensor out, torch::Tensor proj, int64_t col0,
   TORCH_CHECK(nseq >= 1 && state_slots.numel() >= nseq);
   if (rows == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  const bool vec = C % 8 == 0 && col0 % 8 == 0 && proj.stride(0) % 8 == 0 &&
+                   aligned16(proj.data_ptr()) && aligned16(out.data_ptr()) &&
+                   aligned16(cw.data_ptr()) && aligned16(bias.data_ptr()) &&
+                   aligned16(state.data_ptr());
+  if (vec) {
+    const int threads = C / 8 >= 256 ? 256 : 64;
+    dim3 vgrid((unsigned)rows, (unsigned)((C / 8 + threads - 1) / threads));
+    KK_DISPATCH_ACT(proj, {
+      conv_act_vec_kernel<T><<<vgrid, threads, 0, stream>>>(
+          reinterpret_cast<T*>(out.data_ptr()),
+          reinterpret_cast<const T*>(proj.data_ptr()), (long)proj.stride(0),
+          (long)col0, cw.data_ptr<float>(), bias.data_ptr<float>(),
+          state.data_ptr<float>(), positions.data_ptr<int>(),
+          row_seq.data_ptr<int>(), cu_rows.data_ptr<int>(),
+          state_slots.data_ptr<int>(), (int)C, (int)taps, (int)act);
+    });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   dim3 grid((unsigned)rows, (unsigned)((C + 255) / 256));
   KK_DISPATCH_ACT(proj, {
     conv_act_kernel<T><<<grid, 256, 0, stream>>>(

@@ -36,6 +36,51 @@ __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(
   }
 }
 
+// Vector form: a part of at most 8 * 256 * NIT entries, a multiple of 8; the
+// gated values stay in registers between the two passes.
+template <typename T, int NIT>
+__global__ __launch_bounds__(256) void gated_group_rmsnorm_vec_kernel(
+    T* __restrict__ out, const float* __restrict__ y, const T* __restrict__ z,
+    long ldz, const float* __restrict__ w, float eps, int C, int parts) {
+  __shared__ float red[32];
+  const long row = blockIdx.x;
+  const int part = blockIdx.y;
+  const int Cp = C / parts;
+  const int c0 = part * Cp;
+  const float* yr = y + row * (long)C + c0;
+  const T* zr = z + row * ldz + c0;
+  float v[NIT][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int i = (it * 256 + threadIdx.x) * 8;
+    if (i < Cp) {
+      float g[8];
+      ld8(yr + i, v[it]);
+      ld8(zr + i, g);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        v[it][k] *= silu_f(g[k]);
+        ss += v[it][k] * v[it][k];
+      }
+    }
+  }
+  const float2 tot = block_sum2(ss, 0.f, red);
+  const float rs = 1.0f / sqrtf(tot.x / (float)Cp + eps);
+  T* orow = out + row * (long)C + c0;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int i = (it * 256 + threadIdx.x) * 8;
+    if (i < Cp) {
+      float t[8], o[8];
+      ld8(w + c0 + i, t);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) o[k] = v[it][k] * rs * t[k];
+      st8(orow + i, o);
+    }
+  }
+}
+
 void gated_group_rmsnorm(torch::Tensor out, torch::Tensor y, torch::Tensor z,
                          torch::Tensor w, int64_t parts, double eps) {
   check_act(out, "out"); check_act(z, "z");
@@ -50,6 +95,25 @@ void gated_group_rmsnorm(torch::Tensor out, torch::Tensor y, torch::Tensor z,
   if (rows == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
   dim3 grid((unsigned)rows, (unsigned)parts);
+  const int Cp = C / (int)parts;
+  if (Cp % 8 == 0 && Cp <= 8 * 256 * 2 && z.stride(0) % 8 == 0 &&
+      aligned16(out.data_ptr()) && aligned16(y.data_ptr()) &&
+      aligned16(z.data_ptr()) && aligned16(w.data_ptr())) {
+    KK_DISPATCH_ACT(out, {
+      T* op = reinterpret_cast<T*>(out.data_ptr());
+      const T* zp = reinterpret_cast<const T*>(z.data_ptr());
+      if (Cp <= 2048)
+        gated_group_rmsnorm_vec_kernel<T, 1><<<grid, 256, 0, stream>>>(
+            op, y.data_ptr<float>(), zp, (long)z.stride(0),
+            w.data_ptr<float>(), (float)eps, C, (int)parts);
+      else
+        gated_group_rmsnorm_vec_kernel<T, 2><<<grid, 256, 0, stream>>>(
+            op, y.data_ptr<float>(), zp, (long)z.stride(0),
+            w.data_ptr<float>(), (float)eps, C, (int)parts);
+    });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   KK_DISPATCH_ACT(out, {
     gated_group_rmsnorm_kernel<T><<<grid, 256, 0, stream>>>(
         reinterpret_cast<T*>(out.data_ptr()), y.data_ptr<float>(),
@@ -110,6 +174,21 @@ __global__ __launch_bounds__(256) void xielu_kernel(
   stf(out + i, r);
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void xielu_vec_kernel(
+    T* __restrict__ out, const T* __restrict__ z, long total8, float ap,
+    float aq) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  float v[8], r[8];
+  ld8(z + i * 8, v);
+#pragma unroll
+  for (int k = 0; k < 8; ++k)
+    r[k] = v[k] > 0.f ? fmaf(ap * v[k], v[k], 0.5f * v[k])
+                      : fmaf(aq, expm1f(v[k]) - v[k], 0.5f * v[k]);
+  st8(out + i * 8, r);
+}
+
 void xielu(torch::Tensor out, torch::Tensor z, double ap, double aq) {
   check_act(out, "out"); check_act(z, "z");
   TORCH_CHECK(out.is_contiguous() && z.is_contiguous() &&
@@ -118,6 +197,18 @@ void xielu(torch::Tensor out, torch::Tensor z, double ap, double aq) {
   const long total = z.numel();
   if (total == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  if (total % 8 == 0 && aligned16(out.data_ptr()) && aligned16(z.data_ptr())) {
+    const long total8 = total / 8;
+    KK_DISPATCH_ACT(out, {
+      xielu_vec_kernel<T><<<dim3((unsigned)((total8 + 255) / 256)), 256, 0,
+                            stream>>>(
+          reinterpret_cast<T*>(out.data_ptr()),
+          reinterpret_cast<const T*>(z.data_ptr()), total8, (float)ap,
+          (float)aq);
+    });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   KK_DISPATCH_ACT(out, {
     xielu_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0, stream>>>(
         reinterpret_cast<T*>(out.data_ptr()),

@@ -3,10 +3,12 @@
 //   S_t  = exp(-rate_h dt_t) S_(t-1) + dt_t B_t x_t^T        (S: N x P)
 //   y_t  = S_t^T C_t + skip_h x_t
 // One workgroup per (sequence, head). The state matrix stays in registers
-// for the whole portion: thread (p, l) owns rows n = l, l+LN, ... of column
-// p, so a step is NR fused multiply-adds per thread plus a reduction over
-// the LN neighbouring lanes. B, C, x and the step sizes of TT tokens are
-// staged in LDS at a time. All arithmetic is fp32; the state slot is read
+// for the whole portion: thread (p, l) owns the NR consecutive rows
+// n = l NR .. l NR + NR - 1 of column p, so a step is NR fused multiply-adds
+// per thread plus a reduction over the LN neighbouring lanes. B, C, x and
+// the step sizes of TT tokens are staged in LDS at a time; the B and C rows
+// are padded with zeros to LN NR entries, which keeps state rows past N at
+// zero and lets every thread read its share as 16-byte pieces. All arithmetic is fp32; the state slot is read
 // once at the start of the portion (zeros at position 0, whatever the slot
 // held) and written once at its end. A single decoded token is a portion
 // of length one. Tokens are visited in order, so a position's result does
@@ -26,9 +28,10 @@ __global__ __launch_bounds__(1024) void ssm_scan_kernel(
     const int* __restrict__ cu_rows, const int* __restrict__ state_slots,
     int H, int P, int N, int G, int LN) {
   extern __shared__ float sm[];
-  float* sB = sm;                       // [TT][N]
-  float* sC = sB + SSM_TT * N;          // [TT][N]
-  float* sX = sC + SSM_TT * N;          // [TT][P]
+  const int NP = LN * NR;               // padded row of B and C
+  float* sB = sm;                       // [TT][NP]
+  float* sC = sB + SSM_TT * NP;         // [TT][NP]
+  float* sX = sC + SSM_TT * NP;         // [TT][P]
   float* sDT = sX + SSM_TT * P;         // [TT]
   float* sDE = sDT + SSM_TT;            // [TT]
   const int s = blockIdx.x;
@@ -44,12 +47,27 @@ __global__ __launch_bounds__(1024) void ssm_scan_kernel(
   const int p = tid / LN;
   const int l = tid - p * LN;
   const bool live = p < P;
-  float* st = state + (((long)state_slots[s] * H + h) * N) * P;
+  // a column's N state rows are contiguous in the slot: [H, P, N]
+  float* st = state + (((long)state_slots[s] * H + h) * P + (live ? p : 0)) *
+                          (long)N + l * NR;
+  const bool vec4 = (N & 3) == 0;
   float S[NR];
 #pragma unroll
-  for (int k = 0; k < NR; ++k) {
-    const int nn = l + k * LN;
-    S[k] = (live && nn < N && p0 > 0) ? st[(long)nn * P + p] : 0.f;
+  for (int k4 = 0; k4 < NR / 4; ++k4) {
+    const int nn = l * NR + 4 * k4;
+    float4 v = float4{0.f, 0.f, 0.f, 0.f};
+    if (live && p0 > 0) {
+      if (vec4) {
+        if (nn < N) v = *reinterpret_cast<const float4*>(st + 4 * k4);
+      } else {
+        if (nn < N) v.x = st[4 * k4];
+        if (nn + 1 < N) v.y = st[4 * k4 + 1];
+        if (nn + 2 < N) v.z = st[4 * k4 + 2];
+        if (nn + 3 < N) v.w = st[4 * k4 + 3];
+      }
+    }
+    S[4 * k4] = v.x; S[4 * k4 + 1] = v.y;
+    S[4 * k4 + 2] = v.z; S[4 * k4 + 3] = v.w;
   }
   const float bias_h = dt_bias[h];
   const float rate_h = rate[h];
@@ -57,11 +75,11 @@ __global__ __launch_bounds__(1024) void ssm_scan_kernel(
   for (int t0 = 0; t0 < n; t0 += SSM_TT) {
     const int tt = min(SSM_TT, n - t0);
     __syncthreads();
-    for (int i = tid; i < tt * N; i += blockDim.x) {
-      const int t = i / N, nn = i - t * N;
+    for (int i = tid; i < tt * NP; i += blockDim.x) {
+      const int t = i / NP, nn = i - t * NP;
       const T* row = xbc + (row0 + t0 + t) * ldx + inner + (long)g * N + nn;
-      sB[i] = ldf(row);
-      sC[i] = ldf(row + (long)G * N);
+      sB[i] = nn < N ? ldf(row) : 0.f;
+      sC[i] = nn < N ? ldf(row + (long)G * N) : 0.f;
     }
     for (int i = tid; i < tt * P; i += blockDim.x) {
       const int t = i / P, pp = i - t * P;
@@ -78,16 +96,21 @@ __global__ __launch_bounds__(1024) void ssm_scan_kernel(
       const float x = live ? sX[t * P + p] : 0.f;
       const float de = sDE[t];
       const float dx = sDT[t] * x;
-      const float* bt = sB + t * N;
-      const float* ct = sC + t * N;
+      const float4* bt = reinterpret_cast<const float4*>(sB + t * NP + l * NR);
+      const float4* ct = reinterpret_cast<const float4*>(sC + t * NP + l * NR);
       float acc = 0.f;
 #pragma unroll
-      for (int k = 0; k < NR; ++k) {
-        const int nn = l + k * LN;
-        if (nn < N) {
-          S[k] = fmaf(de, S[k], bt[nn] * dx);
-          acc = fmaf(S[k], ct[nn], acc);
-        }
+      for (int k4 = 0; k4 < NR / 4; ++k4) {
+        const float4 b = bt[k4];
+        const float4 c = ct[k4];
+        S[4 * k4 + 0] = fmaf(de, S[4 * k4 + 0], b.x * dx);
+        S[4 * k4 + 1] = fmaf(de, S[4 * k4 + 1], b.y * dx);
+        S[4 * k4 + 2] = fmaf(de, S[4 * k4 + 2], b.z * dx);
+        S[4 * k4 + 3] = fmaf(de, S[4 * k4 + 3], b.w * dx);
+        acc = fmaf(S[4 * k4 + 0], c.x, acc);
+        acc = fmaf(S[4 * k4 + 1], c.y, acc);
+        acc = fmaf(S[4 * k4 + 2], c.z, acc);
+        acc = fmaf(S[4 * k4 + 3], c.w, acc);
       }
       for (int off = LN >> 1; off > 0; off >>= 1)
         acc += __shfl_xor(acc, off, WAVE);
@@ -98,16 +121,24 @@ __global__ __launch_bounds__(1024) void ssm_scan_kernel(
   }
   if (live) {
 #pragma unroll
-    for (int k = 0; k < NR; ++k) {
-      const int nn = l + k * LN;
-      if (nn < N) st[(long)nn * P + p] = S[k];
+    for (int k4 = 0; k4 < NR / 4; ++k4) {
+      const int nn = l * NR + 4 * k4;
+      if (vec4) {
+        if (nn < N)
+          *reinterpret_cast<float4*>(st + 4 * k4) =
+              float4{S[4 * k4], S[4 * k4 + 1], S[4 * k4 + 2], S[4 * k4 + 3]};
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (nn + k < N) st[4 * k4 + k] = S[4 * k4 + k];
+      }
     }
   }
 }
 
 // y [rows, H*P] fp32; xbc [rows, H*P + 2*G*N] = [x | B | C] (stride(1) ==
 // 1); dt [rows, H] (any row stride); dt_bias, rate, skip [H] fp32; state
-// [slots, H, N, P] fp32.
+// [slots, H, P, N] fp32 (a channel's N state rows contiguous).
 void ssm_scan(torch::Tensor y, torch::Tensor xbc, torch::Tensor dt,
               torch::Tensor dt_bias, torch::Tensor rate, torch::Tensor skip,
               torch::Tensor state, torch::Tensor positions,
@@ -127,8 +158,8 @@ void ssm_scan(torch::Tensor y, torch::Tensor xbc, torch::Tensor dt,
               dt.stride(1) == 1 && dt.scalar_type() == xbc.scalar_type());
   TORCH_CHECK(y.dim() == 2 && y.size(0) == rows && y.size(1) == inner);
   TORCH_CHECK(dt_bias.numel() == H && rate.numel() == H && skip.numel() == H);
-  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == N &&
-              state.size(3) == P);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == P &&
+              state.size(3) == N);
   TORCH_CHECK(positions.numel() == rows);
   const long nseq = cu_rows.numel() - 1;
   TORCH_CHECK(nseq >= 1 && state_slots.numel() >= nseq);
@@ -146,7 +177,8 @@ void ssm_scan(torch::Tensor y, torch::Tensor xbc, torch::Tensor dt,
   TORCH_CHECK((long)LN * NR >= N && (long)P * LN <= 1024,
               "ssm_scan: state ", N, " x ", P, " does not fit a workgroup");
   const int threads = (int)((P * LN + 63) / 64 * 64);
-  const size_t lds = (size_t)SSM_TT * (2 * N + P + 2) * sizeof(float);
+  const size_t lds =
+      (size_t)SSM_TT * (2 * (size_t)LN * NR + P + 2) * sizeof(float);
   TORCH_CHECK(lds <= 64 * 1024, "ssm_scan: tile does not fit LDS");
   auto stream = c10::hip::getCurrentHIPStream().stream();
   dim3 grid((unsigned)nseq, (unsigned)H);

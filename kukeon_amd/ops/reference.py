@@ -434,7 +434,7 @@ def conv_act(out, proj, col0: int, cw, bias, state, positions, row_seq,
 def ssm_scan(y, xbc, dt, dt_bias, rate, skip, state, positions, cu_rows,
              state_slots, H: int, P: int, N: int, G: int) -> None:
     """Selective scan, one token after the other. xbc [T, H*P + 2*G*N] =
-    [x | B | C]; dt [T, H] raw step sizes; state [slots, H, N, P] fp32;
+    [x | B | C]; dt [T, H] raw step sizes; state [slots, H, P, N] fp32;
     y [T, H*P] fp32. Per head: S = exp(-rate softplus(dt + dt_bias)) S +
     dt B x^T, y = S^T C + skip x."""
     inner = H * P
@@ -445,7 +445,7 @@ def ssm_scan(y, xbc, dt, dt_bias, rate, skip, state, positions, cu_rows,
         if r1 <= r0 or int(positions[r0]) < 0:
             continue
         slot = int(state_slots[s])
-        S = state[slot].clone()
+        S = state[slot].transpose(1, 2).clone()              # [H, N, P]
         if int(positions[r0]) == 0:
             S.zero_()
         for r in range(r0, r1):
@@ -461,7 +461,7 @@ def ssm_scan(y, xbc, dt, dt_bias, rate, skip, state, positions, cu_rows,
                 (step[:, None] * B)[:, :, None] * x[:, None, :]
             y[r] = ((S * C[:, :, None]).sum(1) +
                     skip[:, None] * x).reshape(inner)
-        state[slot] = S
+        state[slot] = S.transpose(1, 2)
 
 
 def gated_group_rmsnorm(out, y, z, w, groups: int, eps: float) -> None:

@@ -527,12 +527,12 @@ def case_op_sandwich_norm(device, dtype):
         _close(o2, oracle.rms_norm(x.double(), w, 1e-3), dtype, "norm alone")
 
 
-def case_op_conv(device, dtype, taps=4, cuts=((5, 1, 2, 6), (3, 9))):
+def case_op_conv(device, dtype, taps=4, cuts=((5, 1, 2, 6), (3, 9)),
+                 C=37, col0=5, ld=50):
     """Two sequences cut into portions; the portions of a step share one
     launch; slots start out dirty."""
     from kukeon_amd import ops
     g = torch.Generator().manual_seed(taps)
-    C, col0, ld = 37, 5, 50
     act = _act(dtype)
     lens = [sum(c) for c in cuts]
     full = [torch.randn(n, ld, generator=g).to(act) for n in lens]
@@ -592,7 +592,7 @@ def case_op_scan(device, dtype, H=3, P=5, N=7, G=3, cuts=(4, 1, 9, 1, 1)):
         xd, B.repeat_interleave(per, 1), C.repeat_interleave(per, 1),
         dt[:, 1: 1 + H].double(), dt_bias.double(), a_log.double(),
         skip.double())
-    state = torch.full((3, H, N, P), 9.0, device=device)
+    state = torch.full((3, H, P, N), 9.0, device=device)
     got, at = [], 0
     other = torch.randn(1, inner + 2 * G * N, generator=g).to(act)
     for k, n in enumerate(cuts):
@@ -612,21 +612,24 @@ def case_op_scan(device, dtype, H=3, P=5, N=7, G=3, cuts=(4, 1, 9, 1, 1)):
         got.append(y[1:].cpu())
         at += n
     _close(torch.cat(got), want.reshape(T, inner), dtype, "scan outputs")
-    _close(state[2], S, "fp32" if dtype == "fp32" else dtype, "final state")
+    _close(state[2].transpose(1, 2), S, dtype, "final state")
     assert float((state[1] - 9.0).abs().max()) == 0.0
 
 
 def case_op_gated_norm(device, dtype):
     from kukeon_amd import ops
     g = torch.Generator().manual_seed(3)
-    for rows, C, parts in ((4, 24, 3), (2, 7, 1), (3, 600, 2), (1, 5, 5)):
+    for rows, C, parts in ((4, 24, 3), (2, 7, 1), (3, 600, 2), (1, 5, 5),
+                           (3, 4800, 2), (2, 5000, 1)):
         y = torch.randn(rows, C, generator=g) * 2
-        z = torch.randn(rows, C + 4, generator=g).to(_act(dtype))
+        off = 8 if C % 8 == 0 else 2       # aligned rows take vector loads
+        z = torch.randn(rows, C + 2 * off, generator=g).to(_act(dtype))
         w = torch.randn(C, generator=g)
         out = torch.empty(rows, C, dtype=_act(dtype), device=device)
-        ops.gated_group_rmsnorm(out, y.to(device), z.to(device)[:, 2: 2 + C],
-                                w.to(device), parts, 1e-4)
-        v = y.double() * oracle.silu(z[:, 2: 2 + C].double())
+        ops.gated_group_rmsnorm(out, y.to(device),
+                                z.to(device)[:, off: off + C], w.to(device),
+                                parts, 1e-4)
+        v = y.double() * oracle.silu(z[:, off: off + C].double())
         want = oracle.rms_unit(v.view(rows, parts, C // parts), 1e-4).view(
             rows, C) * w.double()
         _close(out, want, dtype, f"gated norm {C}/{parts}")
@@ -635,14 +638,15 @@ def case_op_gated_norm(device, dtype):
 def case_op_activations(device, dtype):
     from kukeon_amd import ops
     g = torch.Generator().manual_seed(4)
-    z = (torch.randn(6, 50, generator=g) * 3).to(_act(dtype))
-    z[0, :4] = torch.tensor([0.0, -0.0, 1e-3, -1e-3]).to(_act(dtype))
-    out = torch.empty_like(z, device=device)
     p, q = 0.3, -0.8
     ap = math.log1p(math.exp(p))
     aq = 0.5 + math.log1p(math.exp(q))
-    ops.xielu(out, z.to(device), ap, aq)
-    _close(out, oracle.xielu(z.double(), p, q), dtype, "xielu")
+    for width in (52, 51):          # whole 16-byte chunks, and not
+        z = (torch.randn(6, width, generator=g) * 3).to(_act(dtype))
+        z[0, :4] = torch.tensor([0.0, -0.0, 1e-3, -1e-3]).to(_act(dtype))
+        out = torch.empty_like(z, device=device)
+        ops.xielu(out, z.to(device), ap, aq)
+        _close(out, oracle.xielu(z.double(), p, q), dtype, "xielu")
     lg = torch.randn(3, 40, generator=g) * 40
     ld = lg.clone().to(device)
     ops.softcap_(ld, 25.0)

@@ -27,6 +27,9 @@ def test_op_sandwich_norm(dtype):
 @pytest.mark.parametrize("taps", [1, 2, 4])
 def test_op_conv(taps, dtype):
     cases.case_op_conv(DEV, dtype, taps=taps)
+    # eight channels per thread
+    cases.case_op_conv(DEV, dtype, taps=taps, C=40, col0=8, ld=64)
+    cases.case_op_conv(DEV, dtype, taps=taps, C=2560, col0=16, ld=2600)
 
 
 @BOTH
