@@ -261,7 +261,8 @@ __global__ __launch_bounds__(256) void latent_attention_vec_kernel(
     int cs_rows, int dims, const int* __restrict__ positions,
     const int* __restrict__ row_seq, const int* __restrict__ block_table,
     int max_blocks, long rows, int H, int dn, int dr, int R, int BS,
-    int window, float scale) {
+    int window, float scale, int NS, float* __restrict__ split_o,
+    float* __restrict__ split_ml) {
   extern __shared__ float sm[];
   const int KW = R + dr;
   float* sq = sm;                          // [HB][KW]
@@ -274,9 +275,18 @@ __global__ __launch_bounds__(256) void latent_attention_vec_kernel(
   const int tid = threadIdx.x;
   const int p = positions[r];
   if (p < 0) {
-    for (int hb = 0; hb < LAT_HB && h0 + hb < H; ++hb)
-      for (int d = tid; d < R; d += blockDim.x)
-        stf(out + ((long)(h0 + hb) * rows + r) * R + d, 0.f);
+    // an inactive row: zeros (from the first split; the merge is told by
+    // a zero sum to write zeros too)
+    for (int hb = 0; hb < LAT_HB && h0 + hb < H; ++hb) {
+      if (NS == 1) {
+        for (int d = tid; d < R; d += blockDim.x)
+          stf(out + ((long)(h0 + hb) * rows + r) * R + d, 0.f);
+      } else if (tid == 0) {
+        float* ml = split_ml + ((r * H + h0 + hb) * NS + blockIdx.z) * 2;
+        ml[0] = -INFINITY;
+        ml[1] = 0.f;
+      }
+    }
     return;
   }
   const int s = row_seq[r];
@@ -305,6 +315,11 @@ __global__ __launch_bounds__(256) void latent_attention_vec_kernel(
   }
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int nkeys = p - lo + 1;
+  // this block's share of the key chunks (all of them when NS == 1)
+  const int nch = (nkeys + LAT_CH - 1) / LAT_CH;
+  const int cps = (nch + NS - 1) / NS;
+  const int key_begin = (int)blockIdx.z * cps * LAT_CH;
+  const int key_end = min(nkeys, ((int)blockIdx.z + 1) * cps * LAT_CH);
   const int per_row = R / 8;               // threads that cover one latent
   const int NG = 256 / per_row;
   const int dg = tid % per_row;
@@ -319,8 +334,8 @@ __global__ __launch_bounds__(256) void latent_attention_vec_kernel(
   }
   const int* bt = block_table + (long)s * max_blocks;
   const int nchunks8 = KW / 8;
-  for (int c0 = 0; c0 < nkeys; c0 += LAT_CH) {
-    const int cn = min(LAT_CH, nkeys - c0);
+  for (int c0 = key_begin; c0 < key_end; c0 += LAT_CH) {
+    const int cn = min(LAT_CH, key_end - c0);
     __syncthreads();
     float sv[LAT_HB];
 #pragma unroll
@@ -393,11 +408,49 @@ __global__ __launch_bounds__(256) void latent_attention_vec_kernel(
     if (h >= H) continue;
     float sum = 0.f;
     for (int g = 0; g < NG; ++g) sum += part[((long)g * LAT_HB + hb) * R + d];
-    // l is the same in every thread; pick it by a uniform chain
-    float lh = l[0];
+    // m and l are the same in every thread; pick them by a uniform chain
+    float lh = l[0], mh = m[0];
 #pragma unroll
-    for (int x = 1; x < LAT_HB; ++x) lh = hb == x ? l[x] : lh;
-    stf(out + ((long)h * rows + r) * R + d, sum / lh);
+    for (int x = 1; x < LAT_HB; ++x) {
+      lh = hb == x ? l[x] : lh;
+      mh = hb == x ? m[x] : mh;
+    }
+    if (NS == 1) {
+      stf(out + ((long)h * rows + r) * R + d, sum / lh);
+    } else {
+      const long u = (r * H + h) * NS + blockIdx.z;
+      split_o[u * R + d] = sum;
+      if (d == 0) {
+        split_ml[u * 2] = mh;
+        split_ml[u * 2 + 1] = lh;
+      }
+    }
+  }
+}
+
+// Folds the key splits of a row: out = sum_z e^(m_z - M) o_z / sum_z
+// e^(m_z - M) l_z, splits in order. A row without keys gives zeros.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_attention_merge_kernel(
+    T* __restrict__ out, const float* __restrict__ split_o,
+    const float* __restrict__ split_ml, long rows, int H, int R, int NS) {
+  const long r = blockIdx.x;
+  const int h = blockIdx.y;
+  const long u0 = (r * H + h) * NS;
+  float M = -INFINITY;
+  for (int z = 0; z < NS; ++z) M = fmaxf(M, split_ml[(u0 + z) * 2]);
+  float L = 0.f;
+  for (int z = 0; z < NS; ++z) {
+    const float mz = split_ml[(u0 + z) * 2];
+    if (mz > -INFINITY) L += __expf(mz - M) * split_ml[(u0 + z) * 2 + 1];
+  }
+  for (int d = threadIdx.x; d < R; d += blockDim.x) {
+    float acc = 0.f;
+    for (int z = 0; z < NS; ++z) {
+      const float mz = split_ml[(u0 + z) * 2];
+      if (mz > -INFINITY) acc += __expf(mz - M) * split_o[(u0 + z) * R + d];
+    }
+    stf(out + ((long)h * rows + r) * R + d, L > 0.f ? acc / L : 0.f);
   }
 }
 
@@ -667,9 +720,30 @@ void latent_attention(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q,
         (int)block_table.size(1), rows, (int)H, (int)dn, (int)dr, R,         \
         (int)cache.size(2), (int)window, (float)scale
   KK_DISPATCH_ACT(q, {
-    if (vec && lds_vec <= 60 * 1024)
-      latent_attention_vec_kernel<T><<<grid, 256, lds_vec, stream>>>(KK_ARGS);
-    else if (R <= 256)
+    if (vec && lds_vec <= 60 * 1024) {
+      // few rows: split every row's keys over several workgroups
+      const long blocks = (long)grid.x * grid.y;
+      int NS = 1;
+      while (NS < 8 && blocks * NS < 1024) NS <<= 1;
+      const long span = window > 0 ? window : cs.size(0);
+      while (NS > 1 && (long)(NS - 1) * LAT_CH >= span) NS >>= 1;
+      if (NS == 1) {
+        latent_attention_vec_kernel<T><<<grid, 256, lds_vec, stream>>>(
+            KK_ARGS, 1, nullptr, nullptr);
+      } else {
+        auto so = torch::empty({rows * H * NS, (long)R},
+                               q.options().dtype(torch::kFloat32));
+        auto sml = torch::empty({rows * H * NS, 2L},
+                                q.options().dtype(torch::kFloat32));
+        latent_attention_vec_kernel<T>
+            <<<dim3(grid.x, grid.y, (unsigned)NS), 256, lds_vec, stream>>>(
+                KK_ARGS, NS, so.data_ptr<float>(), sml.data_ptr<float>());
+        latent_attention_merge_kernel<T>
+            <<<dim3((unsigned)rows, (unsigned)H), 256, 0, stream>>>(
+                reinterpret_cast<T*>(out.data_ptr()), so.data_ptr<float>(),
+                sml.data_ptr<float>(), rows, (int)H, R, NS);
+      }
+    } else if (R <= 256)
       latent_attention_kernel<T, 1><<<grid, 256, lds, stream>>>(KK_ARGS);
     else if (R <= 512)
       latent_attention_kernel<T, 2><<<grid, 256, lds, stream>>>(KK_ARGS);
