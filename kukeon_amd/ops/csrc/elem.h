@@ -59,7 +59,7 @@ template <> struct Raw8<float> {
   }
 };
 
-inline bool aligned16(const void* p) {
+__host__ __device__ inline bool aligned16(const void* p) {
   return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 }
 

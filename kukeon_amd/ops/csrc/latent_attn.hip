@@ -491,7 +491,8 @@ __global__ __launch_bounds__(128) void latent_attention_mfma_kernel(
     const float* __restrict__ cs, int cs_rows, int dims,
     const int* __restrict__ positions, const int* __restrict__ row_seq,
     const int* __restrict__ block_table, int max_blocks, long rows, int H,
-    int dn, int BS, int window, float scale, int HT) {
+    int dn, int BS, int window, float scale, int HT, int NS,
+    float* __restrict__ split_o, float* __restrict__ split_ml) {
   constexpr int KW = R + DR, KST = KW / 32, VST = R / 32, NDT = R / 16;
   constexpr int LDV = R + 8;               // padded LDS row, 16-byte aligned
   extern __shared__ unsigned short lat_lds[];
@@ -506,10 +507,21 @@ __global__ __launch_bounds__(128) void latent_attention_mfma_kernel(
   unsigned short* vl = lat_lds + wave * 16 * LDV;
   bf16_t* orow = out + ((long)(h < H ? h : 0) * rows + r) * R + 4 * g4;
   const int p = positions[r];
+  // with NS > 1 the row's key tiles are shared out over gridDim.y waves
+  // whose partial sums the merge kernel folds
+  float* sml = split_ml + ((r * H + (h < H ? h : 0)) * NS + blockIdx.y) * 2;
+  float* so = split_o + ((r * H + (h < H ? h : 0)) * NS + blockIdx.y) * (long)R +
+              4 * g4;
   if (p < 0) {
-    if (h < H)
-      for (int dt = 0; dt < NDT; ++dt)
-        *reinterpret_cast<uint2*>(orow + dt * 16) = uint2{0u, 0u};
+    if (h < H) {
+      if (NS == 1) {
+        for (int dt = 0; dt < NDT; ++dt)
+          *reinterpret_cast<uint2*>(orow + dt * 16) = uint2{0u, 0u};
+      } else if (g4 == 0) {
+        sml[0] = -INFINITY;
+        sml[1] = 0.f;
+      }
+    }
     return;
   }
   const int s = row_seq[r];
@@ -551,7 +563,11 @@ __global__ __launch_bounds__(128) void latent_attention_mfma_kernel(
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) o[dt] = lat_f32x4_v{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  for (int j0 = lo & ~15; j0 <= p; j0 += 16) {
+  const int t_first = lo >> 4, t_count = (p >> 4) - t_first + 1;
+  const int tps = (t_count + NS - 1) / NS;
+  const int t_begin = t_first + (int)blockIdx.y * tps;
+  const int t_end = min(t_first + t_count, t_begin + tps);
+  for (int j0 = t_begin * 16; j0 < t_end * 16; j0 += 16) {
     // the lane's key, kept inside the visible range for the loads
     int jc = j0 + rc;
     jc = jc < lo ? lo : (jc > p ? p : jc);
@@ -612,6 +628,17 @@ __global__ __launch_bounds__(128) void latent_attention_mfma_kernel(
     }
   }
   if (h >= H) return;
+  if (NS > 1) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      *reinterpret_cast<float4*>(so + dt * 16) =
+          float4{o[dt][0], o[dt][1], o[dt][2], o[dt][3]};
+    if (g4 == 0) {
+      sml[0] = m;
+      sml[1] = l;
+    }
+    return;
+  }
   const float inv = 1.0f / l;
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) {
@@ -634,8 +661,20 @@ static void launch_latent_mfma(torch::Tensor& out, torch::Tensor& q_abs,
   const int HT = (H + 15) / 16;
   const long units = rows * HT;
   const size_t lds = (size_t)2 * 16 * (R + 8) * sizeof(unsigned short);
+  // few rows (a decode step): share every row's key tiles out over up to
+  // 16 waves so that the device fills, and fold the parts afterwards
+  int NS = 1;
+  while (NS < 16 && units * NS < 1024) NS <<= 1;
+  const long span_tiles = ((window > 0 ? window : cs.size(0)) + 15) / 16 + 1;
+  while (NS > 1 && (long)(NS - 1) * 4 >= span_tiles) NS >>= 1;
+  torch::Tensor so, sml;
+  if (NS > 1) {
+    so = torch::empty({rows * H * NS, (long)R},
+                      q.options().dtype(torch::kFloat32));
+    sml = torch::empty({rows * H * NS, 2L}, q.options().dtype(torch::kFloat32));
+  }
   latent_attention_mfma_kernel<R, DR>
-      <<<dim3((unsigned)((units + 1) / 2)), 128, lds, stream>>>(
+      <<<dim3((unsigned)((units + 1) / 2), (unsigned)NS), 128, lds, stream>>>(
           reinterpret_cast<bf16_t*>(out.data_ptr()),
           reinterpret_cast<const bf16_t*>(q_abs.data_ptr()),
           reinterpret_cast<const bf16_t*>(q.data_ptr()), (long)q.stride(0),
@@ -643,7 +682,14 @@ static void launch_latent_mfma(torch::Tensor& out, torch::Tensor& q_abs,
           cs.data_ptr<float>(), (int)cs.size(0), (int)cs.size(1),
           positions.data_ptr<int>(), row_seq.data_ptr<int>(),
           block_table.data_ptr<int>(), (int)block_table.size(1), rows, H, dn,
-          (int)cache.size(2), window, scale, HT);
+          (int)cache.size(2), window, scale, HT, NS,
+          NS > 1 ? so.data_ptr<float>() : nullptr,
+          NS > 1 ? sml.data_ptr<float>() : nullptr);
+  if (NS > 1)
+    latent_attention_merge_kernel<bf16_t>
+        <<<dim3((unsigned)rows, (unsigned)H), 256, 0, stream>>>(
+            reinterpret_cast<bf16_t*>(out.data_ptr()), so.data_ptr<float>(),
+            sml.data_ptr<float>(), rows, H, R, NS);
 }
 
 // sizes the matrix-core form serves
@@ -685,12 +731,12 @@ void latent_attention(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q,
   TORCH_CHECK(lds <= 60 * 1024, "latent_attention: queries do not fit LDS");
   auto stream = c10::hip::getCurrentHIPStream().stream();
   dim3 grid((unsigned)rows, (unsigned)((H + LAT_HB - 1) / LAT_HB));
-  // prompt portions in bf16 at the served sizes: the matrix cores. Few rows
-  // (a decode step) leave them idle, so those stay with the vector form.
+  // bf16 at the served sizes: the matrix cores, for prompt portions and
+  // (with the keys of a row split over several waves) for decoded rows
   if (is_bf16(q) && latent_attention_mfma_supported(R, dr) && dn % 8 == 0 &&
       q.stride(0) % 8 == 0 && aligned16(q.data_ptr()) &&
       aligned16(cache.data_ptr()) && aligned16(q_abs.data_ptr()) &&
-      aligned16(out.data_ptr()) && rows * ((H + 15) / 16) >= 512) {
+      aligned16(out.data_ptr())) {
 #define KK_MFMA(RR, DD)                                                      \
   launch_latent_mfma<RR, DD>(out, q_abs, q, cache, cs, positions, row_seq,   \
                              block_table, rows, (int)H, (int)dn, (int)window, \

@@ -137,6 +137,25 @@ __global__ __launch_bounds__(256) void head_gate_kernel(
   stf(out + i, ldf(o + ((long)h * rows + t) * dv + d) * g);
 }
 
+// 8 values of one head at a time (dv a multiple of 8)
+template <typename T>
+__global__ __launch_bounds__(256) void head_gate_vec_kernel(
+    T* __restrict__ out, const T* __restrict__ o, const T* __restrict__ gate,
+    long ldg, long rows, int H, int dv) {
+  const long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  const long total = rows * H * dv;
+  if (i >= total) return;
+  const int d = (int)(i % dv);
+  const int h = (int)((i / dv) % H);
+  const long t = i / ((long)dv * H);
+  const float g = 1.0f / (1.0f + __expf(-ldf(gate + t * ldg + h)));
+  float v[8];
+  ld8(o + ((long)h * rows + t) * dv + d, v);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) v[k] *= g;
+  st8(out + i, v);
+}
+
 // out [T, H*dv]; o [H, T, dv] contiguous; gate [T, H] (any row stride).
 void head_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate) {
   check_act(out, "out"); check_act(o, "o"); check_act(gate, "gate");
@@ -150,6 +169,18 @@ void head_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate) {
   const long total = rows * H * dv;
   if (total == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  if (dv % 8 == 0 && aligned16(out.data_ptr()) && aligned16(o.data_ptr())) {
+    KK_DISPATCH_ACT(out, {
+      head_gate_vec_kernel<T><<<dim3((unsigned)((total / 8 + 255) / 256)), 256,
+                                0, stream>>>(
+          reinterpret_cast<T*>(out.data_ptr()),
+          reinterpret_cast<const T*>(o.data_ptr()),
+          reinterpret_cast<const T*>(gate.data_ptr()), (long)gate.stride(0),
+          rows, (int)H, (int)dv);
+    });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   KK_DISPATCH_ACT(out, {
     head_gate_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0,
                           stream>>>(

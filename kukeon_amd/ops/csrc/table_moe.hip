@@ -318,8 +318,6 @@ void table_moe(torch::Tensor out, torch::Tensor h, torch::Tensor ids,
   const int top = (int)table.size(1);
   TORCH_CHECK(top >= 1);
   if (rows == 0) return;
-  TORCH_CHECK((size_t)W * 4 <= 64 * 1024 && (size_t)top * ff * 4 <= 64 * 1024,
-              "table_moe: a row does not fit LDS");
   auto act = torch::empty({rows * top, (long)ff}, h.options());
   auto stream = c10::hip::getCurrentHIPStream().stream();
   const int per_block = 4 * MOE_ROWS_PER_WAVE;
@@ -330,6 +328,11 @@ void table_moe(torch::Tensor out, torch::Tensor h, torch::Tensor ids,
                         aligned16(w_up.data_ptr());
   const bool down_major = small && ff % 8 == 0 && aligned16(act.data_ptr()) &&
                           aligned16(w_down.data_ptr());
+  // the token-major kernels stage one row in LDS
+  TORCH_CHECK(up_major || (size_t)W * 4 <= 64 * 1024,
+              "table_moe: an input row does not fit LDS");
+  TORCH_CHECK(down_major || (size_t)top * ff * 4 <= 64 * 1024,
+              "table_moe: a token's expert rows do not fit LDS");
   torch::Tensor part;
   if (down_major || (up_major && W / 8 > MOE_SEG * WAVE))
     part = torch::empty({pairs, (long)std::max(W, ff)},
@@ -416,6 +419,14 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(
   const long r = blockIdx.x;
   const T* src = in + (long)map[r] * W;
   T* dst = out + r * (long)W;
+  if (W % 8 == 0 && aligned16(in) && aligned16(out)) {
+    for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
+      Raw8<T> v;
+      v.load(src + i);
+      *reinterpret_cast<Raw8<T>*>(dst + i) = v;
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < W; i += blockDim.x) dst[i] = src[i];
 }
 
@@ -441,10 +452,23 @@ void gather_rows(torch::Tensor out, torch::Tensor in, torch::Tensor map) {
 template <typename T>
 __global__ __launch_bounds__(256) void relu_square_kernel(T* __restrict__ x,
                                                           long total) {
-  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (i >= total) return;
-  const float v = fmaxf(ldf(x + i), 0.f);
-  stf(x + i, v * v);
+  if (i + 8 <= total && aligned16(x)) {
+    float v[8];
+    ld8(x + i, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      v[k] = fmaxf(v[k], 0.f);
+      v[k] *= v[k];
+    }
+    st8(x + i, v);
+    return;
+  }
+  for (long j = i; j < total && j < i + 8; ++j) {
+    const float v = fmaxf(ldf(x + j), 0.f);
+    stf(x + j, v * v);
+  }
 }
 
 void relu_square_(torch::Tensor x) {
@@ -454,7 +478,7 @@ void relu_square_(torch::Tensor x) {
   if (total == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
   KK_DISPATCH_ACT(x, {
-    relu_square_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0,
+    relu_square_kernel<T><<<dim3((unsigned)((total + 2047) / 2048)), 256, 0,
                             stream>>>(reinterpret_cast<T*>(x.data_ptr()),
                                       total);
   });
@@ -467,6 +491,23 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(
     int W, int top) {
   const long t = blockIdx.x;
   const float share = 1.0f / (float)top;
+  if (W % 8 == 0 && aligned16(in) && aligned16(out)) {
+    for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
+      float acc[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+      for (int k = 0; k < top; ++k) {
+        float v[8];
+        ld8(in + (long)inv[t * top + k] * W + i, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] += v[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] *= share;
+      st8(out + t * (long)W + i, acc);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k)

@@ -651,13 +651,30 @@ def case_op_activations(device, dtype):
     ld = lg.clone().to(device)
     ops.softcap_(ld, 25.0)
     _close(ld, 25.0 * torch.tanh(lg.double() / 25.0), "fp32", "soft cap")
-    o = torch.randn(3, 5, 6, generator=g).to(_act(dtype))
-    gate = torch.randn(5, 3 + 2, generator=g).to(_act(dtype))
-    out = torch.empty(5, 18, dtype=_act(dtype), device=device)
-    ops.head_gate(out, o.to(device), gate.to(device)[:, 1:4])
-    want = (o.double().permute(1, 0, 2) *
-            torch.sigmoid(gate[:, 1:4].double())[:, :, None]).reshape(5, 18)
-    _close(out, want, dtype, "head gate")
+    for dv in (6, 16):
+        o = torch.randn(3, 5, dv, generator=g).to(_act(dtype))
+        gate = torch.randn(5, 3 + 2, generator=g).to(_act(dtype))
+        out = torch.empty(5, 3 * dv, dtype=_act(dtype), device=device)
+        ops.head_gate(out, o.to(device), gate.to(device)[:, 1:4])
+        want = (o.double().permute(1, 0, 2) *
+                torch.sigmoid(gate[:, 1:4].double())[:, :, None]).reshape(
+                    5, 3 * dv)
+        _close(out, want, dtype, "head gate")
+    # rows gathered, squared and folded back (the sorted form of the experts)
+    for W in (24, 21):
+        src = torch.randn(7, W, generator=g).to(_act(dtype))
+        rmap = torch.tensor([3, 3, 0, 6, 1, 2], dtype=torch.int32)
+        got = torch.empty(6, W, dtype=_act(dtype), device=device)
+        ops.gather_rows(got, src.to(device), rmap.to(device))
+        assert torch.equal(got.cpu(), src[rmap.long()])
+        ops.relu_square_(got)
+        _close(got, torch.relu(src[rmap.long()].double()) ** 2, dtype,
+               "relu squared")
+        inv = torch.tensor([[5, 0], [2, 2], [4, 1]], dtype=torch.int32)
+        out = torch.empty(3, W, dtype=_act(dtype), device=device)
+        ops.combine_rows(out, got, inv.to(device))
+        _close(out, got.cpu().double()[inv.long()].mean(1), dtype,
+               "rows folded")
 
 
 def case_op_table_moe(device, dtype, E=5, top=2, W=24, ff=13, V=11, rows=9):
