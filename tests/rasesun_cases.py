@@ -456,14 +456,13 @@ def case_greedy(device, dtype, graphs=False):
             assert out[i][:2] == want[:2], f"request {i}"
 
 
-def case_registry(tmp_path, device, dtype):
-    """A checkpoint folder is found by its architecture name and read."""
+def write_checkpoint(folder, cfg, W):
+    """config.json and model.safetensors (8-byte header length, JSON header,
+    raw data) of a config dictionary and its tensors."""
     import json
+    import os
     import struct
-    from kukeon_amd.models.registry import load_checkpoint
-    cfg = CONFIGS["looped"]()
-    W = weights(cfg, 11)
-    with open(tmp_path / "config.json", "w") as f:
+    with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(cfg, f)
     head, blobs, at = {}, [], 0
     for name, t in W.items():
@@ -475,8 +474,80 @@ def case_registry(tmp_path, device, dtype):
         blobs.append(raw)
         at += len(raw)
     hj = json.dumps(head).encode()
-    with open(tmp_path / "model.safetensors", "wb") as f:
+    with open(os.path.join(folder, "model.safetensors"), "wb") as f:
         f.write(struct.pack("<Q", len(hj)) + hj + b"".join(blobs))
+
+
+def case_trace_runner(tmp_path, device, dtype):
+    """The trace runner as a program: a checkpoint folder, steps on standard
+    input, logits files and `done` lines back. Three requests through a pool
+    sized for two, portions beside single tokens, a request left out of a
+    step."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    cfg = CONFIGS["hybrid"]()
+    W = weights(cfg, 14)
+    model_dir = tmp_path / "model"
+    out_dir = tmp_path / "out"
+    model_dir.mkdir()
+    write_checkpoint(model_dir, cfg, W)
+    prompts = {"a": tokens(cfg, 70, 90), "b": tokens(cfg, 40, 91),
+               "c": tokens(cfg, 33, 92)}
+    want = {k: oracle.forward(cfg, W, p) for k, p in prompts.items()}
+    steps = [[("a", 30), ("b", 1)], [("a", 1), ("b", 38)], [("a", 39)],
+             [("b", 1), ("c", 2)], [("c", 30)], [("c", 1)]]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, os.path.join(root, "bin", "trace_run"), "--model",
+           str(model_dir), "--dtype",
+           "float32" if dtype == "fp32" else "bfloat16", "--out",
+           str(out_dir), "--max-tokens", "128", "--slots", "2", "--device",
+           device]
+    p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                         text=True, cwd=root)
+    at = {k: 0 for k in prompts}
+    try:
+        for n, step in enumerate(steps):
+            entries, end = [], []
+            for k, cnt in step:
+                toks = prompts[k][at[k]: at[k] + cnt]
+                entries.append({"id": k, "tokens": toks,
+                                "want": [0, cnt - 1] if cnt > 1 else [0]})
+                at[k] += cnt
+                if at[k] == len(prompts[k]):
+                    end.append(k)
+            p.stdin.write(json.dumps({"step": n, "entries": entries,
+                                      "end": end}) + "\n")
+            p.stdin.flush()
+            line = p.stdout.readline()
+            while line and line.strip() != "done %d" % n:
+                line = p.stdout.readline()
+            assert line, "the runner ended early"
+            got = np.fromfile(out_dir / ("%d.f32" % n), dtype="<f4").reshape(
+                -1, cfg["vocab"])
+            row = 0
+            for k, cnt in step:
+                a = at[k] - cnt
+                for w in ([0, cnt - 1] if cnt > 1 else [0]):
+                    check(torch.from_numpy(got[row].copy())[None],
+                          want[k][a + w][None], dtype, f"step {n} {k}+{w}")
+                    row += 1
+            assert row == got.shape[0]
+        p.stdin.close()
+        assert p.wait(timeout=60) == 0
+    finally:
+        if p.poll() is None:
+            p.kill()
+
+
+def case_registry(tmp_path, device, dtype):
+    """A checkpoint folder is found by its architecture name and read."""
+    from kukeon_amd.models.registry import load_checkpoint
+    cfg = CONFIGS["looped"]()
+    W = weights(cfg, 11)
+    write_checkpoint(tmp_path, cfg, W)
     mcfg, model = load_checkpoint(str(tmp_path), device=device, dtype=dtype)
     assert mcfg.family == "rasesun" and len(model.runs) == 6
     eng = LLMEngine(model, mcfg, EngineConfig(

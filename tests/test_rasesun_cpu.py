@@ -62,6 +62,10 @@ def test_checkpoint_folder(tmp_path):
     cases.case_registry(tmp_path, DEV, DT)
 
 
+def test_trace_runner(tmp_path):
+    cases.case_trace_runner(tmp_path, DEV, DT)
+
+
 def test_op_sandwich_norm():
     cases.case_op_sandwich_norm(DEV, DT)
 

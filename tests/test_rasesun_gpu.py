@@ -161,3 +161,8 @@ def test_greedy_generation(dtype, graphs):
 @BOTH
 def test_checkpoint_folder(tmp_path, dtype):
     cases.case_registry(tmp_path, DEV, dtype)
+
+
+@BOTH
+def test_trace_runner(tmp_path, dtype):
+    cases.case_trace_runner(tmp_path, DEV, dtype)
