@@ -91,6 +91,20 @@ CONFIGS = {
         layer(latent(heads=3, dim=8, rot_dim=32, rot_dims=12, vdim=8,
                      q_rank=16, kv_rank=128, window=50), dense(48)),
     ], width=48, vocab=40),
+    # no attention at all (no cache pages), and no recurrence at all (no
+    # state), a loop that runs once
+    "only_ssm": lambda: config([
+        layer(ssm(heads=2, vdim=4, state=5, groups=1, conv=3,
+                  norm_groups=2), dense(20)),
+        layer(ssm(heads=1, vdim=8, state=3, groups=1, conv=2,
+                  norm_groups=1), None),
+    ], width=16, vocab=21, loop=(0, 1, 1)),
+    "only_latent": lambda: config([
+        layer(latent(heads=2, dim=4, rot_dim=4, vdim=4, q_rank=6,
+                     kv_rank=8, window=6), moe(3, 2, 8)),
+        layer(latent(heads=1, dim=8, rot_dim=2, vdim=3, q_rank=5,
+                     kv_rank=16, window=300), None),
+    ], width=16, vocab=21),
     # the whole stack looped, attention first, window of one, one tap,
     # no embedding scale, no soft cap
     "looped": lambda: _looped(),
