@@ -120,11 +120,15 @@ class StateSpaceMixer(nn.Module):
         proj = ops.linear(h, self.w_in)
         inner, C = m.inner, m.conv_channels
         xbc = torch.empty(T, C, dtype=h.dtype, device=h.device)
+        # a step of single tokens shifts the slots in the same launch
+        one = meta.max_rows == 1 and T == meta.cu_rows.numel() - 1
         ops.conv_act(xbc, proj, inner, self.conv_w, self.conv_b, conv_state,
                      meta.positions, meta.row_seq, meta.cu_rows,
-                     meta.state_slots, 1)
-        ops.conv_tail_update(conv_state, proj, inner, self.zero_b,
-                             meta.positions, meta.cu_rows, meta.state_slots)
+                     meta.state_slots, 1, one)
+        if not one:
+            ops.conv_tail_update(conv_state, proj, inner, self.zero_b,
+                                 meta.positions, meta.cu_rows,
+                                 meta.state_slots)
         y = torch.empty(T, inner, dtype=torch.float32, device=h.device)
         ops.ssm_scan(y, xbc, proj[:, inner + C:inner + C + m.heads],
                      self.dt_bias, self.rate, self.skip, ssm_state,

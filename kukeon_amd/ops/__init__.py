@@ -478,12 +478,14 @@ def postnorm_residual_rmsnorm(x, y, post_w, w, eps: float, out) -> None:
 
 
 def conv_act(out, proj, col0: int, cw, bias, state, positions, row_seq,
-             cu_rows, state_slots, act: int = 1) -> None:
+             cu_rows, state_slots, act: int = 1,
+             shift_state: bool = False) -> None:
     """Short causal convolution per channel over proj[:, col0:col0+C] with
     carried taps, bias after the sum, then the activation (1: silu, 0:
-    none). Does not touch the state; conv_tail_update shifts it."""
+    none). With `shift_state` (every sequence brings exactly one row) the
+    same launch shifts the state slots; otherwise conv_tail_update does."""
     _recur(proj).conv_act(out, proj, col0, cw, bias, state, positions,
-                          row_seq, cu_rows, state_slots, act)
+                          row_seq, cu_rows, state_slots, act, shift_state)
 
 
 def conv_tail_update(state, proj, col0: int, zero_bias, positions, cu_rows,

@@ -16,7 +16,8 @@ void postnorm_residual_rmsnorm(torch::Tensor x, torch::Tensor y,
 void conv_act(torch::Tensor out, torch::Tensor proj, int64_t col0,
               torch::Tensor cw, torch::Tensor bias, torch::Tensor state,
               torch::Tensor positions, torch::Tensor row_seq,
-              torch::Tensor cu_rows, torch::Tensor state_slots, int64_t act);
+              torch::Tensor cu_rows, torch::Tensor state_slots, int64_t act,
+              bool shift_state);
 void conv_state_update(torch::Tensor state, torch::Tensor proj,
                        torch::Tensor bias, torch::Tensor positions,
                        torch::Tensor cu_rows, torch::Tensor state_slots,

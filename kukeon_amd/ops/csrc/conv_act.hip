@@ -7,7 +7,8 @@
 // read by a new sequence. Taps are summed oldest first whatever the
 // portion's length, so a position's value does not depend on how the
 // prompt was cut. The slot itself is shifted afterwards by
-// conv_state_update.
+// conv_state_update, or by this kernel when every sequence brings exactly
+// one row (a decode step): then a thread owns its channels of the slot.
 #include "elem.h"
 
 namespace kukeon {
@@ -16,9 +17,10 @@ template <typename T>
 __global__ __launch_bounds__(256) void conv_act_kernel(
     T* __restrict__ out, const T* __restrict__ proj, long ldp, long col0,
     const float* __restrict__ cw, const float* __restrict__ bias,
-    const float* __restrict__ state, const int* __restrict__ positions,
+    float* __restrict__ state, const int* __restrict__ positions,
     const int* __restrict__ row_seq, const int* __restrict__ cu_rows,
-    const int* __restrict__ state_slots, int C, int taps, int act) {
+    const int* __restrict__ state_slots, int C, int taps, int act,
+    int shift) {
   const long r = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
@@ -28,7 +30,7 @@ __global__ __launch_bounds__(256) void conv_act_kernel(
   const long row0 = cu_rows[s];
   const int i = (int)(r - row0);
   const int back = taps - 1;
-  const float* st = state + (long)state_slots[s] * back * C;
+  float* st = state + (long)state_slots[s] * back * C;
   float acc = 0.f;
   for (int j = 0; j < taps; ++j) {
     const int src = i - back + j;
@@ -40,6 +42,12 @@ __global__ __launch_bounds__(256) void conv_act_kernel(
   acc += bias[c];
   if (act == 1) acc = acc / (1.0f + __expf(-acc));
   stf(out + r * (long)C + c, acc);
+  if (shift && back > 0) {
+    // the sequence's only row: this thread owns its channel of the slot
+    for (int k = 0; k + 1 < back; ++k)
+      st[(long)k * C + c] = st[(long)(k + 1) * C + c];
+    st[(long)(back - 1) * C + c] = ldf(proj + r * ldp + col0 + c);
+  }
 }
 
 // Vector form: 8 consecutive channels per thread, every tap one 16-byte (bf16)
@@ -48,9 +56,10 @@ template <typename T>
 __global__ __launch_bounds__(256) void conv_act_vec_kernel(
     T* __restrict__ out, const T* __restrict__ proj, long ldp, long col0,
     const float* __restrict__ cw, const float* __restrict__ bias,
-    const float* __restrict__ state, const int* __restrict__ positions,
+    float* __restrict__ state, const int* __restrict__ positions,
     const int* __restrict__ row_seq, const int* __restrict__ cu_rows,
-    const int* __restrict__ state_slots, int C, int taps, int act) {
+    const int* __restrict__ state_slots, int C, int taps, int act,
+    int shift) {
   const long r = blockIdx.x;
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   if (c >= C) return;
@@ -60,7 +69,7 @@ __global__ __launch_bounds__(256) void conv_act_vec_kernel(
   const long row0 = cu_rows[s];
   const int i = (int)(r - row0);
   const int back = taps - 1;
-  const float* st = state + (long)state_slots[s] * back * C;
+  float* st = state + (long)state_slots[s] * back * C;
   float acc[8];
 #pragma unroll
   for (int k = 0; k < 8; ++k) acc[k] = 0.f;
@@ -82,6 +91,15 @@ __global__ __launch_bounds__(256) void conv_act_vec_kernel(
     if (act == 1) acc[k] = acc[k] / (1.0f + __expf(-acc[k]));
   }
   st8(out + r * (long)C + c, acc);
+  if (shift && back > 0) {
+    float u[8];
+    for (int k = 0; k + 1 < back; ++k) {
+      ld8(st + (long)(k + 1) * C + c, u);
+      st8(st + (long)k * C + c, u);
+    }
+    ld8(proj + r * ldp + col0 + c, u);
+    st8(st + (long)(back - 1) * C + c, u);
+  }
 }
 
 // out [rows, C] contiguous; proj [rows, ld] (stride(1) == 1) read at
@@ -90,7 +108,8 @@ __global__ __launch_bounds__(256) void conv_act_vec_kernel(
 void conv_act(torch::Tensor out, torch::Tensor proj, int64_t col0,
               torch::Tensor cw, torch::Tensor bias, torch::Tensor state,
               torch::Tensor positions, torch::Tensor row_seq,
-              torch::Tensor cu_rows, torch::Tensor state_slots, int64_t act) {
+              torch::Tensor cu_rows, torch::Tensor state_slots, int64_t act,
+              bool shift_state) {
   check_act(proj, "proj");
   check_f32(cw, "cw"); check_f32(bias, "bias"); check_f32(state, "state");
   check_i32(positions, "positions"); check_i32(row_seq, "row_seq");
@@ -109,6 +128,9 @@ void conv_act(torch::Tensor out, torch::Tensor proj, int64_t col0,
   const long nseq = cu_rows.numel() - 1;
   TORCH_CHECK(nseq >= 1 && state_slots.numel() >= nseq);
   if (rows == 0) return;
+  TORCH_CHECK(!shift_state || rows == nseq,
+              "the state is shifted in place only when every sequence brings "
+              "one row");
   auto stream = c10::hip::getCurrentHIPStream().stream();
   const bool vec = C % 8 == 0 && col0 % 8 == 0 && proj.stride(0) % 8 == 0 &&
                    aligned16(proj.data_ptr()) && aligned16(out.data_ptr()) &&
@@ -124,7 +146,8 @@ void conv_act(torch::Tensor out, torch::Tensor proj, int64_t col0,
           (long)col0, cw.data_ptr<float>(), bias.data_ptr<float>(),
           state.data_ptr<float>(), positions.data_ptr<int>(),
           row_seq.data_ptr<int>(), cu_rows.data_ptr<int>(),
-          state_slots.data_ptr<int>(), (int)C, (int)taps, (int)act);
+          state_slots.data_ptr<int>(), (int)C, (int)taps, (int)act,
+          (int)shift_state);
     });
     HIP_CHECK_KERNEL();
     return;
@@ -137,7 +160,8 @@ void conv_act(torch::Tensor out, torch::Tensor proj, int64_t col0,
         (long)col0, cw.data_ptr<float>(), bias.data_ptr<float>(),
         state.data_ptr<float>(), positions.data_ptr<int>(),
         row_seq.data_ptr<int>(), cu_rows.data_ptr<int>(),
-        state_slots.data_ptr<int>(), (int)C, (int)taps, (int)act);
+        state_slots.data_ptr<int>(), (int)C, (int)taps, (int)act,
+        (int)shift_state);
   });
   HIP_CHECK_KERNEL();
 }

@@ -403,7 +403,8 @@ def postnorm_residual_rmsnorm(x, y, post_w, w, eps: float, out) -> None:
 
 
 def conv_act(out, proj, col0: int, cw, bias, state, positions, row_seq,
-             cu_rows, state_slots, act: int = 1) -> None:
+             cu_rows, state_slots, act: int = 1,
+             shift_state: bool = False) -> None:
     """out = act(causal_conv(proj[:, col0:col0+C]) + bias) per sequence;
     the taps before a portion come from the state slot (zeros before the
     sequence start). cw [taps, C] with the newest tap last. act 1 = silu."""
@@ -429,6 +430,10 @@ def conv_act(out, proj, col0: int, cw, bias, state, positions, row_seq,
         if act == 1:
             y = y * torch.sigmoid(y)
         out[r0:r1] = y.to(out.dtype)
+        if shift_state and back:
+            assert n == 1
+            slot = int(state_slots[s])
+            state[slot] = torch.cat([state[slot], u], 0)[-back:]
 
 
 def ssm_scan(y, xbc, dt, dt_bias, rate, skip, state, positions, cu_rows,
