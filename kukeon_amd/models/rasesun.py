@@ -148,8 +148,10 @@ def rasesun_bench(width=4096, layers=8, heads=32, ff=14336, vocab=128256,
                                 rot_dims=64, rot_base=10000.0)
         else:
             kind = "mamba2"
-            mix = StateSpaceCfg(heads=2 * width // 64, vdim=64, state=128,
-                                groups=8, conv=4, norm_groups=8)
+            ssm_heads = max(1, 2 * width // 64)
+            parts = 8 if ssm_heads % 8 == 0 else 1
+            mix = StateSpaceCfg(heads=ssm_heads, vdim=64, state=128,
+                                groups=parts, conv=4, norm_groups=parts)
         if i % 2:
             mlp = FFCfg("moe", max(8, ff // top // 8 * 8), experts=experts,
                         top=top)

@@ -470,6 +470,89 @@ def case_greedy(device, dtype, graphs=False):
             assert out[i][:2] == want[:2], f"request {i}"
 
 
+def assert_greedy(cfg, W, prompt, got, what=""):
+    """Every generated token is the plain model's best one, up to the
+    rounding of the logits to bfloat16 that the sampler works on."""
+    toks = list(prompt)
+    for i, t in enumerate(got):
+        lg = oracle.forward(cfg, W, toks)[-1]
+        best = float(lg.max())
+        assert float(lg[t]) >= best - abs(best) * 2.0 ** -7, \
+            f"{what}: token {i} is {t}, the plain model says " \
+            f"{int(lg.argmax())}"
+        toks.append(t)
+
+
+def _generate(eng, kv, prompt, n):
+    sp = SamplingParams(temperature=0.0, max_new_tokens=n)
+    eng.add_request(kv, prompt, sp)
+    out = []
+    while eng.has_work():
+        for o in eng.step():
+            out.extend(o.new_tokens)
+    return out
+
+
+def case_multi_turn(device, dtype):
+    """A session's second turn continues from its pages and state slots; an
+    idle session whose pages and slot were taken away is rebuilt from its
+    history."""
+    cfg = CONFIGS["hybrid"]()
+    W = weights(cfg, 15)
+    eng = make_engine(cfg, W, device, dtype, blocks=12, slots=2, max_len=64,
+                      poison=False, decode_microbatch=2)
+    a, b = SequenceKV(4), SequenceKV(4)
+    p1, p2, p3 = tokens(cfg, 9, 60), tokens(cfg, 5, 61), tokens(cfg, 30, 62)
+    t1 = _generate(eng, a, p1, 4)
+    assert_greedy(cfg, W, p1, t1, "first turn")
+    t2 = _generate(eng, a, p2, 3)
+    assert_greedy(cfg, W, p1 + t1 + p2, t2, "second turn")
+    assert a.num_tokens > 0 and a.state_slot >= 0
+    # b needs more pages than are left: a's pages and slot are taken
+    tb = _generate(eng, b, p3, 4)
+    assert_greedy(cfg, W, p3, tb, "other session")
+    assert a.num_tokens == 0 and a.state_slot < 0 and a.history
+    eng.free_sequence(b)
+    t3 = _generate(eng, a, [7, 3], 3)
+    assert len(t1) == 4 and len(t2) == 3 and len(tb) == 4 and len(t3) == 3
+    assert_greedy(cfg, W, p1 + t1 + p2 + t2 + [7, 3], t3, "rebuilt session")
+
+
+def case_modelhub(device):
+    """The serving daemon's model server with this family: sessions over the
+    unix socket, two turns on one session, greedy tokens as the plain model
+    gives them."""
+    import uuid
+    from kukeon_amd.serve.server import ModelhubClient, ModelhubServer
+    cfg = CONFIGS["hybrid"]()
+    W = weights(cfg, 16)
+    mcfg = RasesunConfig.from_json(cfg)
+    model = RasesunModel(mcfg, device=device, dtype="fp32", tensors=W,
+                         max_position=128)
+    ecfg = EngineConfig(block_size=4, max_model_len=128, max_sessions=4,
+                        state_slots=4, num_kv_blocks=64, use_graphs=False)
+    sock = f"/tmp/mh-{uuid.uuid4().hex[:10]}.sock"
+    hub = ModelhubServer(model, mcfg, ecfg, sock, device=device)
+    hub.start()
+    try:
+        c = ModelhubClient(sock, timeout=120)
+        p1, p2 = tokens(cfg, 6, 70), tokens(cfg, 3, 71)
+        r1 = c.generate("s", p1, max_new_tokens=4, temperature=0.0)
+        assert len(r1["tokens"]) == 4
+        assert_greedy(cfg, W, p1, r1["tokens"], "first turn")
+        r2 = c.generate("s", p2, max_new_tokens=3, temperature=0.0)
+        assert len(r2["tokens"]) == 3
+        assert_greedy(cfg, W, p1 + r1["tokens"] + p2, r2["tokens"],
+                      "second turn")
+        rb = c.generate("t", p2, max_new_tokens=2, temperature=0.0)
+        assert len(rb["tokens"]) == 2
+        assert_greedy(cfg, W, p2, rb["tokens"], "other session")
+        assert c.call("stats")["sessions"] == 2
+        c.close()
+    finally:
+        hub.stop()
+
+
 def write_checkpoint(folder, cfg, W):
     """config.json and model.safetensors (8-byte header length, JSON header,
     raw data) of a config dictionary and its tensors."""

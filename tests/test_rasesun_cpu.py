@@ -62,6 +62,24 @@ def test_checkpoint_folder(tmp_path):
     cases.case_registry(tmp_path, DEV, DT)
 
 
+def test_multi_turn_and_eviction():
+    cases.case_multi_turn(DEV, DT)
+
+
+def test_modelhub_serves_the_family():
+    cases.case_modelhub(DEV)
+
+
+def test_presets_build_through_the_registry():
+    from kukeon_amd.models import registry
+    assert "rasesun-8b-like" in registry.preset_names()
+    cfg = registry.preset("tiny-rasesun")
+    model = registry.build_model(cfg, "cpu", dtype="fp32")
+    assert model.family == "rasesun" and len(model.runs) == 4
+    kinds = [type(L.mixer).__name__ for L in model.layers]
+    assert kinds.count("LatentAttention") == 1
+
+
 def test_trace_runner(tmp_path):
     cases.case_trace_runner(tmp_path, DEV, DT)
 

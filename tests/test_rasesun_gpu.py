@@ -158,6 +158,10 @@ def test_greedy_generation(dtype, graphs):
     cases.case_greedy(DEV, dtype, graphs=graphs)
 
 
+def test_multi_turn_and_eviction():
+    cases.case_multi_turn(DEV, "fp32")
+
+
 @BOTH
 def test_checkpoint_folder(tmp_path, dtype):
     cases.case_registry(tmp_path, DEV, dtype)
